@@ -7,6 +7,7 @@ tiny_llm/pipeline/pipeline.cpp:30-31); here config.json chooses.
 """
 from __future__ import annotations
 
+import inspect
 import json
 import os
 from typing import Any, Callable, Dict, Mapping, Tuple
@@ -37,24 +38,32 @@ def known_architectures():
 
 
 def architecture_name(raw: Mapping[str, Any]) -> str:
+    """`architectures` (a list, its first entry counts, or a string) or `architecture` (a string)."""
     arch = raw.get("architectures")
     if isinstance(arch, (list, tuple)) and arch:
         return str(arch[0])
     if isinstance(arch, str):
         return arch
+    if isinstance(raw.get("architecture"), str):
+        return raw["architecture"]
     raise UnknownArchitecture(
         "config.json has no `architectures`; known: " + ", ".join(known_architectures()))
 
 
-def resolve(raw: Mapping[str, Any]):
-    """Raw config.json dict -> (typed config, ModelSpec)."""
+def resolve(raw: Mapping[str, Any], tensor_shapes: Mapping[str, Any] = None):
+    """Raw config.json dict -> (typed config, ModelSpec).  `tensor_shapes` ({name: shape} of the
+    checkpoint, optional) goes to readers that take it: an architecture may leave a size to the
+    shapes of its tensors."""
     name = architecture_name(raw)
     if name not in _ARCHITECTURES:
         raise UnknownArchitecture(
             f"no model registered for architecture {name!r}; known: "
             + ", ".join(known_architectures()))
     read_config, build_spec = _ARCHITECTURES[name]
-    cfg = read_config(raw)
+    if tensor_shapes is not None and "shapes" in inspect.signature(read_config).parameters:
+        cfg = read_config(raw, shapes=tensor_shapes)
+    else:
+        cfg = read_config(raw)
     spec = build_spec(cfg)
     spec.validate()
     return cfg, spec

@@ -1,0 +1,242 @@
+// The gated delta rule with one decay per head and key channel, as a recurrence over a state
+// S [dim, vdim] per request and head:
+//     S <- diag(g_t) S;  u = beta_t (v_t - S^T k_t);  S <- S + k_t u^T;  o_t = S^T q_t
+// and what surrounds it: short causal convolutions with SiLU on q, k and v (their last taps - 1
+// inputs are state as well), unit vectors q and k, the decay g = exp(-exp(A_log) softplus(a + dt_bias)),
+// and the per-head norm with its gate on the way out.  The state, and everything that enters the
+// recurrence, is float32 in both precisions.
+//
+// Per request the state is ONE row of float32: [S of every head: heads x dim x vdim | the
+// convolutions' last inputs: channels x (taps - 1), oldest first].
+#include "common.h"
+
+namespace {
+
+constexpr int kPrepThreads = 128;
+constexpr int kPrepWaves = kPrepThreads / TL_WAVE;
+constexpr int kMaxDim = 256;      // key channels a head may have
+
+__device__ __forceinline__ float silu(float x) { return x / (1.f + expf(-x)); }
+__device__ __forceinline__ float softplus(float x) { return x > 20.f ? x : log1pf(expf(x)); }
+
+// Input m of channel c (column `col` of the projections) of the request whose tokens of this step
+// start at row t0: m >= 0 is row t0 + m of this step, m < 0 reaches back into the saved inputs.
+template <typename T>
+__device__ __forceinline__ float conv_input(const T* __restrict__ p, int64_t p_stride, int t0, int m, int col,
+                                            const float* __restrict__ saved, int taps) {
+  return m >= 0 ? to_f32(p[(int64_t)(t0 + m) * p_stride + col]) : saved[(taps - 1) + m];
+}
+
+template <typename T>
+__device__ __forceinline__ float conv_silu(const T* __restrict__ p, int64_t p_stride, int t0, int n, int col,
+                                           const float* __restrict__ saved, const float* __restrict__ w, int taps) {
+  float acc = 0.f;
+  for (int b = 0; b < taps; ++b) acc = fmaf(w[taps - 1 - b], conv_input(p, p_stride, t0, n - b, col, saved, taps), acc);
+  return silu(acc);
+}
+
+// One workgroup per (token, head).  Row t of `p` holds [q (kv_heads x dim) | k (kv_heads x dim) |
+// v (heads x vdim)] from column conv_off on, and beta's pre-activation at column b_off + head;
+// row t of `a` holds the decay's pre-activation at column head * dim + i.
+template <typename T>
+__global__ __launch_bounds__(kPrepThreads) void delta_prepare_kernel(
+    const T* __restrict__ p, int64_t p_stride, int conv_off, int b_off, const float* __restrict__ a, int64_t a_stride,
+    const float* __restrict__ conv_w, const float* __restrict__ a_log, const float* __restrict__ dt_bias,
+    const float* __restrict__ state, int64_t state_stride, int64_t saved_off, const int32_t* __restrict__ req_of_token,
+    const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ state_slots, float* __restrict__ qn,
+    float* __restrict__ kn, float* __restrict__ vc, float* __restrict__ beta, float* __restrict__ decay, int heads,
+    int kv_heads, int dim, int vdim, int taps, float q_scale) {
+  __shared__ float qs[kMaxDim], ks[kMaxDim], red[kPrepWaves];
+  const int t = blockIdx.x, h = blockIdx.y;
+  const int r = req_of_token[t];
+  const int t0 = cu_seqlens[r], t1 = cu_seqlens[r + 1];
+  const int64_t base = (int64_t)t * heads + h;
+  if (t < t0 || t >= t1) {            // a padding row of a captured step: finite stand-ins, never read
+    for (int i = threadIdx.x; i < dim; i += kPrepThreads) qn[base * dim + i] = kn[base * dim + i] = decay[base * dim + i] = 0.f;
+    for (int j = threadIdx.x; j < vdim; j += kPrepThreads) vc[base * vdim + j] = 0.f;
+    if (threadIdx.x == 0) beta[base] = 0.f;
+    return;
+  }
+  const int n = t - t0;
+  const int kh = h / (heads / kv_heads);
+  const float* saved = state + (int64_t)state_slots[r] * state_stride + saved_off;
+  const int q_ch = kh * dim, k_ch = kv_heads * dim + kh * dim, v_ch = 2 * kv_heads * dim + h * vdim;
+  float sq = 0.f, sk = 0.f;
+  for (int i = threadIdx.x; i < dim; i += kPrepThreads) {
+    const float q = conv_silu(p, p_stride, t0, n, conv_off + q_ch + i, saved + (int64_t)(q_ch + i) * (taps - 1),
+                              conv_w + (int64_t)(q_ch + i) * taps, taps);
+    const float k = conv_silu(p, p_stride, t0, n, conv_off + k_ch + i, saved + (int64_t)(k_ch + i) * (taps - 1),
+                              conv_w + (int64_t)(k_ch + i) * taps, taps);
+    qs[i] = q;
+    ks[i] = k;
+    sq += q * q;
+    sk += k * k;
+  }
+  sq = block_sum<kPrepWaves>(sq, red);
+  sk = block_sum<kPrepWaves>(sk, red);
+  const float rq = q_scale / sqrtf(sq + 1e-6f), rk = 1.f / sqrtf(sk + 1e-6f);
+  const float rate = expf(a_log[h]);
+  for (int i = threadIdx.x; i < dim; i += kPrepThreads) {
+    qn[base * dim + i] = qs[i] * rq;
+    kn[base * dim + i] = ks[i] * rk;
+    const float pre = a[(int64_t)t * a_stride + h * dim + i] + dt_bias[h * dim + i];
+    decay[base * dim + i] = expf(-rate * softplus(pre));
+  }
+  for (int j = threadIdx.x; j < vdim; j += kPrepThreads)
+    vc[base * vdim + j] = conv_silu(p, p_stride, t0, n, conv_off + v_ch + j, saved + (int64_t)(v_ch + j) * (taps - 1),
+                                    conv_w + (int64_t)(v_ch + j) * taps, taps);
+  if (threadIdx.x == 0) beta[base] = 1.f / (1.f + expf(-to_f32(p[(int64_t)t * p_stride + b_off + h])));
+}
+
+// The convolutions' saved inputs after a step: the last taps - 1 of (what was saved, this step's
+// inputs).  One thread per (request, channel); it reads all it needs before it writes.
+constexpr int kMaxTaps = 16;
+template <typename T>
+__global__ void conv_state_update_kernel(const T* __restrict__ p, int64_t p_stride, int conv_off, int channels,
+                                         float* __restrict__ state, int64_t state_stride, int64_t saved_off,
+                                         const int32_t* __restrict__ cu_seqlens,
+                                         const int32_t* __restrict__ state_slots, int taps) {
+  const int r = blockIdx.y;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  const int t0 = cu_seqlens[r], n = cu_seqlens[r + 1] - t0;
+  if (c >= channels || n <= 0) return;
+  float* saved = state + (int64_t)state_slots[r] * state_stride + saved_off + (int64_t)c * (taps - 1);
+  float next[kMaxTaps];
+#pragma unroll
+  for (int i = 0; i < kMaxTaps; ++i)
+    if (i < taps - 1) next[i] = conv_input(p, p_stride, t0, n - (taps - 1) + i, conv_off + c, saved, taps);
+#pragma unroll
+  for (int i = 0; i < kMaxTaps; ++i)
+    if (i < taps - 1) saved[i] = next[i];
+}
+
+// The recurrence.  One wave per (request, head, 64 value columns); lane j keeps column j of S in
+// registers and walks the request's tokens of this step in order.  q, k and the decay of a token
+// are the same for all lanes.
+template <int DIM>
+__global__ __launch_bounds__(TL_WAVE) void delta_recurrence_kernel(
+    const float* __restrict__ qn, const float* __restrict__ kn, const float* __restrict__ vc,
+    const float* __restrict__ beta, const float* __restrict__ decay, float* __restrict__ state, int64_t state_stride,
+    const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ state_slots, float* __restrict__ out,
+    int heads, int dim, int vdim) {
+  const int r = blockIdx.x, h = blockIdx.y;
+  const int col = blockIdx.z * TL_WAVE + threadIdx.x;
+  const int t0 = cu_seqlens[r], t1 = cu_seqlens[r + 1];
+  if (t1 <= t0 || col >= vdim) return;        // a padding request owns no state
+  float* S_mem = state + (int64_t)state_slots[r] * state_stride + (int64_t)h * dim * vdim + col;
+  float S[DIM];
+#pragma unroll
+  for (int i = 0; i < DIM; ++i) S[i] = i < dim ? S_mem[(int64_t)i * vdim] : 0.f;
+  for (int t = t0; t < t1; ++t) {
+    const int64_t base = (int64_t)t * heads + h;
+    const float* __restrict__ k = kn + base * dim;
+    const float* __restrict__ q = qn + base * dim;
+    const float* __restrict__ g = decay + base * dim;
+    float sk = 0.f;
+#pragma unroll
+    for (int i = 0; i < DIM; ++i)
+      if (i < dim) {
+        S[i] *= g[i];
+        sk = fmaf(S[i], k[i], sk);
+      }
+    const float u = beta[base] * (vc[base * vdim + col] - sk);
+    float o = 0.f;
+#pragma unroll
+    for (int i = 0; i < DIM; ++i)
+      if (i < dim) {
+        S[i] = fmaf(k[i], u, S[i]);
+        o = fmaf(S[i], q[i], o);
+      }
+    out[base * vdim + col] = o;
+  }
+#pragma unroll
+  for (int i = 0; i < DIM; ++i)
+    if (i < dim) S_mem[(int64_t)i * vdim] = S[i];
+}
+
+// z[t, h, :] = w * o[t, h, :] / sqrt(mean(o[t, h, :]^2) + eps) * sigmoid(gate[t, h, :]); one wave per (t, h).
+template <typename T>
+__global__ __launch_bounds__(TL_WAVE) void head_norm_gate_kernel(const float* __restrict__ o,
+                                                                 const float* __restrict__ w,
+                                                                 const float* __restrict__ gate, int64_t gate_stride,
+                                                                 T* __restrict__ z, int heads, int vdim, float eps) {
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const float* src = o + ((int64_t)t * heads + h) * vdim;
+  float ss = 0.f;
+  for (int j = lane; j < vdim; j += TL_WAVE) ss += src[j] * src[j];
+  ss = wave_sum(ss);
+  const float r = 1.f / sqrtf(ss / (float)vdim + eps);
+  const float* gp = gate + (int64_t)t * gate_stride + (int64_t)h * vdim;
+  T* dst = z + ((int64_t)t * heads + h) * vdim;
+  for (int j = lane; j < vdim; j += TL_WAVE) dst[j] = from_f32<T>(src[j] * r * w[j] / (1.f + expf(-gp[j])));
+}
+
+}  // namespace
+
+#define TL_DISPATCH_T(dtype, ...)                 \
+  if ((dtype) == 0) { using T = float; __VA_ARGS__ } \
+  else if ((dtype) == 1) { using T = bf16_t; __VA_ARGS__ } \
+  else return TL_ERR_ARG;
+
+extern "C" {
+
+int tl_delta_prepare(const void* p, int64_t p_stride, int conv_off, int b_off, const float* a, int64_t a_stride,
+                     const float* conv_w, const float* a_log, const float* dt_bias, const float* state,
+                     int64_t state_stride, int64_t saved_off, const int32_t* req_of_token, const int32_t* cu_seqlens,
+                     const int32_t* state_slots, float* qn, float* kn, float* vc, float* beta, float* decay,
+                     int n_tokens, int heads, int kv_heads, int dim, int vdim, int taps, float q_scale, int dtype,
+                     hipStream_t stream) {
+  if (n_tokens <= 0) return TL_OK;
+  if (heads <= 0 || heads > 65535 || kv_heads <= 0 || heads % kv_heads || dim <= 0 || dim > kMaxDim || vdim <= 0 ||
+      taps < 1 || taps > kMaxTaps)
+    return TL_ERR_ARG;
+  dim3 g(n_tokens, heads), b(kPrepThreads);
+  TL_DISPATCH_T(dtype, hipLaunchKernelGGL(delta_prepare_kernel<T>, g, b, 0, stream, (const T*)p, p_stride, conv_off,
+                                          b_off, a, a_stride, conv_w, a_log, dt_bias, state, state_stride, saved_off,
+                                          req_of_token, cu_seqlens, state_slots, qn, kn, vc, beta, decay, heads,
+                                          kv_heads, dim, vdim, taps, q_scale);)
+  return tl_launch_status();
+}
+
+int tl_conv_state_update(const void* p, int64_t p_stride, int conv_off, int channels, float* state,
+                         int64_t state_stride, int64_t saved_off, const int32_t* cu_seqlens,
+                         const int32_t* state_slots, int n_requests, int taps, int dtype, hipStream_t stream) {
+  if (n_requests <= 0 || taps <= 1) return TL_OK;
+  if (channels <= 0 || taps > kMaxTaps || n_requests > 65535) return TL_ERR_ARG;
+  dim3 g((channels + 255) / 256, n_requests), b(256);
+  TL_DISPATCH_T(dtype, hipLaunchKernelGGL(conv_state_update_kernel<T>, g, b, 0, stream, (const T*)p, p_stride,
+                                          conv_off, channels, state, state_stride, saved_off, cu_seqlens, state_slots,
+                                          taps);)
+  return tl_launch_status();
+}
+
+int tl_delta_recurrence(const float* qn, const float* kn, const float* vc, const float* beta, const float* decay,
+                        float* state, int64_t state_stride, const int32_t* cu_seqlens, const int32_t* state_slots,
+                        float* out, int n_requests, int heads, int dim, int vdim, hipStream_t stream) {
+  if (n_requests <= 0) return TL_OK;
+  if (heads <= 0 || heads > 65535 || dim <= 0 || dim > kMaxDim || vdim <= 0 || (vdim + 63) / 64 > 65535)
+    return TL_ERR_ARG;
+  dim3 g(n_requests, heads, (vdim + TL_WAVE - 1) / TL_WAVE), b(TL_WAVE);
+#define TL_REC(D)                                                                                                    \
+  hipLaunchKernelGGL(delta_recurrence_kernel<D>, g, b, 0, stream, qn, kn, vc, beta, decay, state, state_stride,      \
+                     cu_seqlens, state_slots, out, heads, dim, vdim)
+  if (dim <= 16) TL_REC(16);
+  else if (dim <= 32) TL_REC(32);
+  else if (dim <= 64) TL_REC(64);
+  else if (dim <= 128) TL_REC(128);
+  else TL_REC(256);
+#undef TL_REC
+  return tl_launch_status();
+}
+
+int tl_head_norm_gate(const float* o, const float* w, const float* gate, int64_t gate_stride, void* z, int n_tokens,
+                      int heads, int vdim, float eps, int dtype, hipStream_t stream) {
+  if (n_tokens <= 0) return TL_OK;
+  if (heads <= 0 || heads > 65535 || vdim <= 0) return TL_ERR_ARG;
+  dim3 g(n_tokens, heads), b(TL_WAVE);
+  TL_DISPATCH_T(dtype, hipLaunchKernelGGL(head_norm_gate_kernel<T>, g, b, 0, stream, o, w, gate, gate_stride, (T*)z,
+                                          heads, vdim, eps);)
+  return tl_launch_status();
+}
+
+}  // extern "C"

@@ -1,0 +1,119 @@
+// Kernels around a sublayer whose norm sits on its OUTPUT: x += scale * w * y / rms(y), the copy
+// of the residual stream in the engine's element type that the next sublayer's products read, a
+// gated unit with clamped inputs, and the soft cap of the logits.
+//
+// The residual stream, the norm's statistics and its weight are float32 in both precisions.
+#include "common.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWaves = kThreads / TL_WAVE;
+
+// x[t] += scale * w * y[t] / sqrt(mean(y[t]^2) + eps); copy[t] = x[t] in TC (optional).
+// One workgroup per row.  `w` is the norm's effective weight, `scale` (optional) a factor per channel.
+template <typename TC>
+__global__ void norm_scale_add_kernel(const float* __restrict__ y, const float* __restrict__ w,
+                                      const float* __restrict__ scale, float* __restrict__ x,
+                                      TC* __restrict__ copy, int hidden, float eps) {
+  __shared__ float red[kWaves];
+  const float* src = y + (int64_t)blockIdx.x * hidden;
+  float* dst = x + (int64_t)blockIdx.x * hidden;
+  float ss = 0.f;
+  for (int j = threadIdx.x; j < hidden; j += kThreads) {
+    const float v = src[j];
+    ss += v * v;
+  }
+  ss = block_sum<kWaves>(ss, red);
+  const float r = 1.f / sqrtf(ss / (float)hidden + eps);
+  for (int j = threadIdx.x; j < hidden; j += kThreads) {
+    float v = src[j] * r * w[j];
+    if (scale) v *= scale[j];
+    const float s = dst[j] + v;
+    dst[j] = s;
+    if (copy) copy[(int64_t)blockIdx.x * hidden + j] = from_f32<TC>(s);
+  }
+}
+
+template <typename TO>
+__global__ void cast_rows_kernel(const float* __restrict__ x, TO* __restrict__ out, int64_t total) {
+  const int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (i < total) out[i] = from_f32<TO>(x[i]);
+}
+
+// z[t, j] = g * sigmoid(alpha * g) * (u + shift), g = min(gate_up[t, j], limit),
+// u = clamp(gate_up[t, inter + j], -limit, limit).
+template <typename T>
+__global__ void clamped_glu_kernel(const T* __restrict__ gate_up, T* __restrict__ z, int64_t total, int inter,
+                                   int64_t in_stride, float limit, float alpha, float shift) {
+  const int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (i >= total) return;
+  const int64_t t = i / inter;
+  const int j = (int)(i - t * inter);
+  const float g = fminf(to_f32(gate_up[t * in_stride + j]), limit);
+  const float u = fminf(fmaxf(to_f32(gate_up[t * in_stride + inter + j]), -limit), limit);
+  z[i] = from_f32<T>(g / (1.f + expf(-alpha * g)) * (u + shift));
+}
+
+__global__ void softcap_kernel(float* __restrict__ x, int64_t total, float cap) {
+  const int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (i < total) x[i] = cap * tanhf(x[i] / cap);
+}
+
+}  // namespace
+
+extern "C" {
+
+// copy_dtype: 0 float32, 1 bfloat16; copy and scale may be null.
+int tl_norm_scale_add(const float* y, const float* w, const float* scale, float* x, void* copy, int n_rows,
+                      int hidden, float eps, int copy_dtype, hipStream_t stream) {
+  if (n_rows <= 0) return TL_OK;
+  if (hidden <= 0) return TL_ERR_ARG;
+  dim3 g(n_rows), b(kThreads);
+  if (copy_dtype == 1)
+    hipLaunchKernelGGL(norm_scale_add_kernel<bf16_t>, g, b, 0, stream, y, w, scale, x, (bf16_t*)copy, hidden, eps);
+  else if (copy_dtype == 0)
+    hipLaunchKernelGGL(norm_scale_add_kernel<float>, g, b, 0, stream, y, w, scale, x, (float*)copy, hidden, eps);
+  else
+    return TL_ERR_ARG;
+  return tl_launch_status();
+}
+
+int tl_cast_rows(const float* x, void* out, int64_t total, int out_dtype, hipStream_t stream) {
+  if (total <= 0) return TL_OK;
+  dim3 g((unsigned)ceil_div64(total, kThreads)), b(kThreads);
+  if (out_dtype == 1)
+    hipLaunchKernelGGL(cast_rows_kernel<bf16_t>, g, b, 0, stream, x, (bf16_t*)out, total);
+  else if (out_dtype == 0)
+    hipLaunchKernelGGL(cast_rows_kernel<float>, g, b, 0, stream, x, (float*)out, total);
+  else
+    return TL_ERR_ARG;
+  return tl_launch_status();
+}
+
+int tl_clamped_glu(const void* gate_up, void* z, int n_rows, int inter, int64_t in_stride, float limit, float alpha,
+                   float shift, int dtype, hipStream_t stream) {
+  if (n_rows <= 0) return TL_OK;
+  if (inter <= 0 || in_stride < 2 * (int64_t)inter) return TL_ERR_ARG;
+  const int64_t total = (int64_t)n_rows * inter;
+  dim3 g((unsigned)ceil_div64(total, kThreads)), b(kThreads);
+  if (dtype == 0)
+    hipLaunchKernelGGL(clamped_glu_kernel<float>, g, b, 0, stream, (const float*)gate_up, (float*)z, total, inter,
+                       in_stride, limit, alpha, shift);
+  else if (dtype == 1)
+    hipLaunchKernelGGL(clamped_glu_kernel<bf16_t>, g, b, 0, stream, (const bf16_t*)gate_up, (bf16_t*)z, total, inter,
+                       in_stride, limit, alpha, shift);
+  else
+    return TL_ERR_ARG;
+  return tl_launch_status();
+}
+
+int tl_softcap(float* x, int64_t total, float cap, hipStream_t stream) {
+  if (total <= 0) return TL_OK;
+  if (!(cap > 0.f)) return TL_ERR_ARG;
+  hipLaunchKernelGGL(softcap_kernel, dim3((unsigned)ceil_div64(total, kThreads)), dim3(kThreads), 0, stream, x, total,
+                     cap);
+  return tl_launch_status();
+}
+
+}  // extern "C"

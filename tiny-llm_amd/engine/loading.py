@@ -10,7 +10,7 @@ from ..cache import CacheManager
 from ..config import EngineConfig, resolve, read_config_json
 from ..kernels import library
 from ..models.decoder import Decoder
-from ..weights import init_random_weights, load_weights
+from ..weights import Checkpoint, init_random_weights, load_weights
 from .step import ModelRunner
 
 
@@ -26,16 +26,19 @@ def require_gpu(device: int = 0) -> torch.device:
     return torch.device(f"cuda:{device}")
 
 
-def build_decoder(config: Mapping, dtype: str, device) -> tuple:
-    cfg, spec = resolve(config)
+def build_decoder(config: Mapping, dtype: str, device, tensor_shapes: Optional[Mapping] = None) -> tuple:
+    cfg, spec = resolve(config, tensor_shapes)
     return cfg, Decoder(spec, dtype=dtype, device=device)
 
 
 def load_model(model_path: str, engine: EngineConfig):
-    """config.json chooses the model class; weights come from the folder's safetensors."""
+    """config.json chooses the model class; weights come from the folder's safetensors (whose
+    headers also give the sizes that an architecture leaves to its tensors' shapes)."""
     device = require_gpu(engine.device)
-    cfg, dec = build_decoder(read_config_json(model_path), engine.dtype, device)
-    load_weights(dec, model_path)
+    ckpt = Checkpoint(model_path)
+    shapes = {n: ckpt.info(n)[1] for n in ckpt.names()}
+    cfg, dec = build_decoder(read_config_json(model_path), engine.dtype, device, shapes)
+    load_weights(dec, ckpt)
     return cfg, dec
 
 

@@ -1059,3 +1059,275 @@ def decode_advance(tokens: torch.Tensor, positions: torch.Tensor, seq_lens: torc
                                     _ptr(history), _ptr(step), c_int(R), c_int(G),
                                     c_int(block_tables[0].shape[1] if G else 1), c_int(block_size),
                                     c_int(history.numel() // R), slots_arr, tables_arr, _stream()), "decode_advance")
+
+
+# ------------------------------------------------- sublayers with the norm on their output
+def _f32_vec(t: Optional[torch.Tensor], n: int, what: str) -> None:
+    if t is not None and not (t.dtype == torch.float32 and t.is_contiguous() and t.numel() == n):
+        _fail(f"{what} must be contiguous float32 with {n} elements")
+
+
+def _i32(*tensors) -> None:
+    for t in tensors:
+        if not (t.dtype == torch.int32 and t.is_contiguous()):
+            _fail("index tensors must be contiguous int32")
+
+
+def norm_scale_add(y: torch.Tensor, weight: torch.Tensor, eps: float, x: torch.Tensor,
+                   scale: Optional[torch.Tensor] = None, copy: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x += scale * weight * y / sqrt(mean(y^2) + eps), all float32; `copy` (optional, float32 or
+    bfloat16, x's shape) receives the new x.  `weight` is the norm's effective weight."""
+    _dev(y, weight, x, scale, copy)
+    if not (y.dtype == torch.float32 and x.dtype == torch.float32 and y.dim() == 2 and y.is_contiguous()
+            and x.is_contiguous() and x.shape == y.shape):
+        _fail("norm_scale_add takes contiguous float32 [T, H] for the sublayer's output and the residual stream")
+    T, H = y.shape
+    _f32_vec(weight, H, "the norm's weight")
+    _f32_vec(scale, H, "the channel scale")
+    if copy is not None and not (copy.is_contiguous() and copy.shape == x.shape):
+        _fail("the copy of the residual stream must be contiguous with its shape")
+    _check(_lib().tl_norm_scale_add(_ptr(y), _ptr(weight), _ptr(scale), _ptr(x), _ptr(copy), c_int(T), c_int(H),
+                                    c_float(eps), c_int(_dt(copy) if copy is not None else 0), _stream()),
+           "norm_scale_add")
+    return x
+
+
+def cast_rows(x: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out = x (float32) in out's element type."""
+    _dev(x, out)
+    if not (x.dtype == torch.float32 and x.is_contiguous() and out.is_contiguous() and out.shape == x.shape):
+        _fail("cast_rows takes contiguous operands of one shape, the input in float32")
+    _check(_lib().tl_cast_rows(_ptr(x), _ptr(out), c_int64(x.numel()), c_int(_dt(out)), _stream()), "cast_rows")
+    return out
+
+
+def clamped_glu(gate_up: torch.Tensor, out: torch.Tensor, limit: float, alpha: float, shift: float) -> torch.Tensor:
+    """out[t, j] = g * sigmoid(alpha * g) * (u + shift) with g = min(gate_up[t, j], limit) and
+    u = clamp(gate_up[t, I + j], -limit, limit)."""
+    _dev(gate_up, out)
+    _rows_2d(gate_up, "gate_up")
+    T, I = out.shape
+    if not (gate_up.shape[0] == T and gate_up.shape[1] >= 2 * I and out.dtype == gate_up.dtype and out.is_contiguous()):
+        _fail("clamped_glu: gate_up is [T, >= 2I], the output contiguous [T, I] of the same type")
+    _check(_lib().tl_clamped_glu(_ptr(gate_up), _ptr(out), c_int(T), c_int(I), c_int64(gate_up.stride(0)),
+                                 c_float(limit), c_float(alpha), c_float(shift), c_int(_dt(out)), _stream()),
+           "clamped_glu")
+    return out
+
+
+def softcap(logits: torch.Tensor, cap: float) -> torch.Tensor:
+    """logits <- cap * tanh(logits / cap), in place (float32)."""
+    _dev(logits)
+    if not (logits.dtype == torch.float32 and logits.is_contiguous() and cap > 0):
+        _fail("softcap takes contiguous float32 logits and a positive cap")
+    _check(_lib().tl_softcap(_ptr(logits), c_int64(logits.numel()), c_float(cap), _stream()), "softcap")
+    return logits
+
+
+# ---------------------------------------------------------- attention over cached latents
+LATENT_MAX_RANK = 512       # latent size the attention kernel takes (csrc/latent_attention.hip)
+LATENT_MAX_QUERY = 1024     # latent size + rotated dims
+
+
+def check_latent_sizes(kv_rank: int, rot: int) -> None:
+    if not (0 < kv_rank <= LATENT_MAX_RANK and 0 <= rot and rot % 2 == 0 and kv_rank + rot <= LATENT_MAX_QUERY):
+        _fail(f"latent attention takes latents of up to {LATENT_MAX_RANK} and an even number of rotated "
+              f"dims, together at most {LATENT_MAX_QUERY}; got {kv_rank} and {rot}")
+
+
+def latent_prepare(d: torch.Tensor, q_off: int, q_rank: int, w_q: torch.Tensor, eps: float, cq: torch.Tensor,
+                   kv_off: int = 0, kv_rank: int = 0, rot: int = 0, rdims: int = 0,
+                   w_kv: Optional[torch.Tensor] = None,
+                   positions: Optional[torch.Tensor] = None, cos: Optional[torch.Tensor] = None,
+                   sin: Optional[torch.Tensor] = None, slots: Optional[torch.Tensor] = None,
+                   latent: Optional[torch.Tensor] = None, rope: Optional[torch.Tensor] = None) -> None:
+    """Row t of d holds the down projections.  cq[t] = w_q * unit_rms(d[t, q_off : q_off + q_rank]);
+    with kv_rank > 0 also latent[slots[t]] = w_kv * unit_rms(d[t, kv_off : kv_off + kv_rank]) and
+    rope[slots[t]] = the next `rot` columns, the first `rdims` of them rotated by the angle tables' row
+    positions[t] (pairs (i, i + rdims/2)).  latent / rope are the paged tensors [blocks, block_size, width]."""
+    _dev(d, w_q, cq, w_kv, positions, cos, sin, slots, latent, rope)
+    _rows_2d(d, "projections")
+    T = d.shape[0]
+    _f32_vec(w_q, q_rank, "the query latent's norm weight")
+    if not (cq.dtype == d.dtype and cq.is_contiguous() and tuple(cq.shape) == (T, q_rank)
+            and 0 <= q_off and q_off + q_rank <= d.shape[1]):
+        _fail("latent_prepare: the query latent must be contiguous [T, q_rank] of the projections' type")
+    if kv_rank > 0:
+        _f32_vec(w_kv, kv_rank, "the latent's norm weight")
+        _i32(positions, slots)
+        if not (kv_off >= 0 and kv_off + kv_rank + rot <= d.shape[1] and positions.numel() == T and slots.numel() == T):
+            _fail("latent_prepare: columns or per-token tensors do not fit")
+        if not (latent.dtype == d.dtype and latent.is_contiguous() and latent.shape[-1] == kv_rank):
+            _fail("latent_prepare: the latent cache must be contiguous [..., kv_rank] of the projections' type")
+        if rot:
+            if not (rope.dtype == d.dtype and rope.is_contiguous() and rope.shape[-1] == rot
+                    and rope.numel() // rot == latent.numel() // kv_rank):
+                _fail("latent_prepare: the rotated-key cache must be contiguous [..., rot] with the latent cache's slots")
+            if not (cos.dtype == torch.float32 and sin.dtype == torch.float32 and cos.is_contiguous()
+                    and sin.is_contiguous() and cos.shape == sin.shape and cos.shape[1] == rdims // 2
+                    and 0 < rdims <= rot and rdims % 2 == 0):
+                _fail("latent_prepare: angle tables are float32 [positions, rdims / 2]")
+    _check(_lib().tl_latent_prepare(_ptr(d), c_int64(d.stride(0)), c_int(q_off), c_int(q_rank), c_int(kv_off),
+                                    c_int(kv_rank), c_int(rot), c_int(rdims if kv_rank > 0 else 0), _ptr(w_q), _ptr(w_kv),
+                                    c_float(eps), _ptr(positions),
+                                    _ptr(cos), _ptr(sin), _ptr(slots), _ptr(cq), _ptr(latent), _ptr(rope), c_int(T),
+                                    c_int(_dt(d)), _stream()), "latent_prepare")
+
+
+def rotate_into(q: torch.Tensor, heads: int, head_width: int, in_off: int, rot: int, rdims: int,
+                positions: torch.Tensor,
+                cos: torch.Tensor, sin: torch.Tensor, out: torch.Tensor, out_off: int) -> torch.Tensor:
+    """out[t, h, out_off : out_off + rot] (float32) = the dims in_off : in_off + rot of head h of
+    row t of q, the first `rdims` of them rotated by the angle tables' row positions[t] (pairs
+    (i, i + rdims/2)), the others as they are."""
+    _dev(q, positions, cos, sin, out)
+    _rows_2d(q, "rotate_into input")
+    _i32(positions)
+    T = q.shape[0]
+    if not (q.shape[1] >= heads * head_width and out.dtype == torch.float32 and out.is_contiguous() and out.dim() == 3
+            and out.shape[0] == T and out.shape[1] == heads and positions.numel() == T
+            and cos.dtype == torch.float32 and sin.dtype == torch.float32 and cos.is_contiguous()
+            and sin.is_contiguous() and cos.shape == sin.shape and cos.shape[1] == rdims // 2
+            and 0 < rdims <= rot and rdims % 2 == 0):
+        _fail("rotate_into: shapes do not fit")
+    _check(_lib().tl_rotate_into(_ptr(q), c_int64(q.stride(0)), c_int(head_width), c_int(in_off), c_int(rot),
+                                 c_int(rdims), c_int(heads), _ptr(positions), _ptr(cos), _ptr(sin), _ptr(out), c_int(out.shape[2]),
+                                 c_int(out_off), c_int(T), c_int(_dt(q)), _stream()), "rotate_into")
+    return out
+
+
+def latent_attention(qa: torch.Tensor, latent: torch.Tensor, rope: Optional[torch.Tensor], block_tables: torch.Tensor,
+                     req_of_token: torch.Tensor, positions: torch.Tensor, out: torch.Tensor, scale: float,
+                     gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """qa float32 [T, heads, kv_rank + rot] = [W_uk^T q_unrotated | q_rotated]; latent / rope the paged
+    tensors [blocks, block_size, kv_rank] / [blocks, block_size, rot].  out[t, h] = sigmoid(gate[t, h])
+    * sum_j softmax_j((qa[t, h] . [latent_j | rope_j]) * scale) latent_j over the request's positions
+    j <= positions[t].  gate [T, heads] may be a view with a row stride."""
+    _dev(qa, latent, rope, block_tables, req_of_token, positions, out, gate)
+    _i32(block_tables, req_of_token, positions)
+    T, H, W = qa.shape
+    kv_rank = latent.shape[-1]
+    rot = W - kv_rank
+    check_latent_sizes(kv_rank, rot)
+    if not (qa.dtype == torch.float32 and qa.is_contiguous() and latent.dim() == 3 and latent.is_contiguous()
+            and block_tables.dim() == 2 and req_of_token.numel() == T and positions.numel() == T):
+        _fail("latent_attention: queries are contiguous float32 [T, heads, kv_rank + rot], the cache [blocks, block_size, kv_rank]")
+    if rot and not (rope is not None and rope.dtype == latent.dtype and rope.is_contiguous()
+                    and tuple(rope.shape) == (*latent.shape[:2], rot)):
+        _fail("latent_attention: the rotated-key cache must be [blocks, block_size, rot] of the cache's type")
+    if not (out.dtype == latent.dtype and out.is_contiguous() and tuple(out.shape) == (T, H, kv_rank)):
+        _fail("latent_attention: the output is contiguous [T, heads, kv_rank] of the cache's type")
+    if gate is not None and not (gate.dtype == latent.dtype and gate.dim() == 2 and gate.stride(1) == 1
+                                 and tuple(gate.shape) == (T, H)):
+        _fail("latent_attention: the gate is [T, heads] of the cache's type")
+    _check(_lib().tl_latent_attention(_ptr(qa), _ptr(latent), _ptr(rope), _ptr(block_tables),
+                                      c_int(block_tables.shape[1]), _ptr(req_of_token), _ptr(positions), _ptr(gate),
+                                      c_int64(gate.stride(0) if gate is not None else 0), _ptr(out), c_int(T),
+                                      c_int(H), c_int(kv_rank), c_int(rot), c_int(latent.shape[1]), c_float(scale),
+                                      c_int(_dt(latent)), _stream()), "latent_attention")
+    return out
+
+
+# ------------------------------------------------------------------ gated delta rule
+DELTA_MAX_DIM = 256     # key channels of a head (csrc/delta_rule.hip)
+DELTA_MAX_TAPS = 16
+
+
+def check_delta_sizes(heads: int, kv_heads: int, dim: int, vdim: int, taps: int) -> None:
+    if not (heads > 0 and kv_heads > 0 and heads % kv_heads == 0 and 0 < dim <= DELTA_MAX_DIM and vdim > 0
+            and 1 <= taps <= DELTA_MAX_TAPS):
+        _fail(f"delta rule: heads must be a multiple of kv heads, key channels at most {DELTA_MAX_DIM}, "
+              f"taps at most {DELTA_MAX_TAPS}; got {heads}/{kv_heads} heads, {dim} x {vdim}, {taps} taps")
+
+
+def delta_prepare(p: torch.Tensor, conv_off: int, b_off: int, a: torch.Tensor, conv_w: torch.Tensor,
+                  a_log: torch.Tensor, dt_bias: torch.Tensor, state: torch.Tensor, saved_off: int,
+                  req_of_token: torch.Tensor, cu_seqlens: torch.Tensor, state_slots: torch.Tensor, qn: torch.Tensor,
+                  kn: torch.Tensor, vc: torch.Tensor, beta: torch.Tensor, decay: torch.Tensor, heads: int,
+                  kv_heads: int, dim: int, vdim: int, taps: int, q_scale: float) -> None:
+    """What enters the recurrence, per token and head, in float32: q and k after their causal
+    convolution and SiLU as unit vectors (q times q_scale), v after its convolution and SiLU, beta =
+    sigmoid(p[t, b_off + h]) and decay = exp(-exp(a_log[h]) * softplus(a[t, h * dim + i] + dt_bias)).
+    Row t of p holds [q | k | v] from column conv_off on; inputs before a request's first token of the
+    step come from its state row, at saved_off."""
+    _dev(p, a, conv_w, a_log, dt_bias, state, req_of_token, cu_seqlens, state_slots, qn, kn, vc, beta, decay)
+    check_delta_sizes(heads, kv_heads, dim, vdim, taps)
+    _rows_2d(p, "projections")
+    _rows_2d(a, "decay pre-activations")
+    _i32(req_of_token, cu_seqlens, state_slots)
+    T = p.shape[0]
+    channels = 2 * kv_heads * dim + heads * vdim
+    _f32_vec(conv_w, channels * taps, "convolution taps")
+    _f32_vec(a_log, heads, "A_log")
+    _f32_vec(dt_bias, heads * dim, "dt_bias")
+    if not (a.dtype == torch.float32 and a.shape[0] == T and a.shape[1] >= heads * dim
+            and conv_off >= 0 and conv_off + channels <= p.shape[1] and 0 <= b_off and b_off + heads <= p.shape[1]):
+        _fail("delta_prepare: columns do not fit")
+    if not (state.dtype == torch.float32 and state.dim() == 2 and state.is_contiguous()
+            and saved_off + channels * (taps - 1) <= state.shape[1] and req_of_token.numel() == T):
+        _fail("delta_prepare: the state is contiguous float32 [slots, row] with room for the saved inputs")
+    for t, n in ((qn, T * heads * dim), (kn, T * heads * dim), (vc, T * heads * vdim), (beta, T * heads),
+                 (decay, T * heads * dim)):
+        _f32_vec(t, n, "delta_prepare outputs")
+    _check(_lib().tl_delta_prepare(_ptr(p), c_int64(p.stride(0)), c_int(conv_off), c_int(b_off), _ptr(a),
+                                   c_int64(a.stride(0)), _ptr(conv_w), _ptr(a_log), _ptr(dt_bias), _ptr(state),
+                                   c_int64(state.stride(0)), c_int64(saved_off), _ptr(req_of_token), _ptr(cu_seqlens),
+                                   _ptr(state_slots), _ptr(qn), _ptr(kn), _ptr(vc), _ptr(beta), _ptr(decay), c_int(T),
+                                   c_int(heads), c_int(kv_heads), c_int(dim), c_int(vdim), c_int(taps),
+                                   c_float(q_scale), c_int(_dt(p)), _stream()), "delta_prepare")
+
+
+def conv_state_update(p: torch.Tensor, conv_off: int, channels: int, state: torch.Tensor, saved_off: int,
+                      cu_seqlens: torch.Tensor, state_slots: torch.Tensor, taps: int) -> None:
+    """The saved inputs of the convolutions after this step: per request and channel the last
+    taps - 1 of (what was saved, the step's inputs), oldest first."""
+    _dev(p, state, cu_seqlens, state_slots)
+    _rows_2d(p, "projections")
+    _i32(cu_seqlens, state_slots)
+    R = state_slots.numel()
+    if not (state.dtype == torch.float32 and state.dim() == 2 and state.is_contiguous() and cu_seqlens.numel() == R + 1
+            and saved_off + channels * (taps - 1) <= state.shape[1] and conv_off + channels <= p.shape[1]
+            and 1 <= taps <= DELTA_MAX_TAPS):
+        _fail("conv_state_update: shapes do not fit")
+    _check(_lib().tl_conv_state_update(_ptr(p), c_int64(p.stride(0)), c_int(conv_off), c_int(channels), _ptr(state),
+                                       c_int64(state.stride(0)), c_int64(saved_off), _ptr(cu_seqlens),
+                                       _ptr(state_slots), c_int(R), c_int(taps), c_int(_dt(p)), _stream()),
+           "conv_state_update")
+
+
+def delta_recurrence(qn: torch.Tensor, kn: torch.Tensor, vc: torch.Tensor, beta: torch.Tensor, decay: torch.Tensor,
+                     state: torch.Tensor, cu_seqlens: torch.Tensor, state_slots: torch.Tensor, out: torch.Tensor,
+                     heads: int, dim: int, vdim: int) -> torch.Tensor:
+    """Walks every request's tokens of this step through S <- diag(g) S; u = beta (v - S^T k);
+    S <- S + k u^T; o = S^T q, with S [heads, dim, vdim] at the start of the request's state row."""
+    _dev(qn, kn, vc, beta, decay, state, cu_seqlens, state_slots, out)
+    _i32(cu_seqlens, state_slots)
+    R = state_slots.numel()
+    T = beta.numel() // heads
+    for t, n in ((qn, T * heads * dim), (kn, T * heads * dim), (vc, T * heads * vdim), (beta, T * heads),
+                 (decay, T * heads * dim), (out, T * heads * vdim)):
+        _f32_vec(t, n, "delta_recurrence operands")
+    if not (state.dtype == torch.float32 and state.dim() == 2 and state.is_contiguous()
+            and heads * dim * vdim <= state.shape[1] and cu_seqlens.numel() == R + 1 and 0 < dim <= DELTA_MAX_DIM):
+        _fail("delta_recurrence: the state is contiguous float32 [slots, >= heads * dim * vdim]")
+    _check(_lib().tl_delta_recurrence(_ptr(qn), _ptr(kn), _ptr(vc), _ptr(beta), _ptr(decay), _ptr(state),
+                                      c_int64(state.stride(0)), _ptr(cu_seqlens), _ptr(state_slots), _ptr(out),
+                                      c_int(R), c_int(heads), c_int(dim), c_int(vdim), _stream()), "delta_recurrence")
+    return out
+
+
+def head_norm_gate(o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, out: torch.Tensor, heads: int,
+                   vdim: int, eps: float) -> torch.Tensor:
+    """out[t, h, :] = weight * o[t, h, :] / sqrt(mean(o[t, h, :]^2) + eps) * sigmoid(gate[t, h, :]);
+    o float32 [T, heads * vdim], gate float32 [T, heads * vdim] (a view with a row stride is fine)."""
+    _dev(o, weight, gate, out)
+    T = out.shape[0]
+    _f32_vec(o, T * heads * vdim, "head_norm_gate input")
+    _f32_vec(weight, vdim, "the head norm's weight")
+    if not (gate.dtype == torch.float32 and gate.dim() == 2 and gate.stride(1) == 1
+            and tuple(gate.shape) == (T, heads * vdim) and out.is_contiguous() and tuple(out.shape) == (T, heads * vdim)):
+        _fail("head_norm_gate: gate and output are [T, heads * vdim]")
+    _check(_lib().tl_head_norm_gate(_ptr(o), _ptr(weight), _ptr(gate), c_int64(gate.stride(0)), _ptr(out), c_int(T),
+                                    c_int(heads), c_int(vdim), c_float(eps), c_int(_dt(out)), _stream()),
+           "head_norm_gate")
+    return out

@@ -1,2 +1,2 @@
-from . import llama  # noqa: F401  (registers LlamaForCausalLM)
+from . import llama, lufazen  # noqa: F401  (register LlamaForCausalLM, Lufazen)
 from .decoder import Decoder

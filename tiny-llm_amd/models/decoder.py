@@ -36,7 +36,10 @@ class Layer:
             raise ValueError(f"layer {spec.prefix}: arrangement {spec.block!r} has no role {unknown}; "
                              f"it takes {sorted(roles)}")
         self.by_role: Dict[str, Part] = {}
+        optional = getattr(arrangement, "optional", ())
         for role, category in roles.items():
+            if role not in spec.parts and role in optional:
+                continue
             if role not in spec.parts:
                 raise ValueError(f"layer {spec.prefix}: arrangement {spec.block!r} needs a part for role {role!r}")
             ps = spec.parts[role]

@@ -173,18 +173,24 @@ class FeedForward(Part):
         raise NotImplementedError
 
 
+class ChannelScale(Part):
+    """One learned factor per channel (a sublayer's result times a vector)."""
+
+
 class Block:
     """An arrangement of a layer's parts around the residual stream.
 
     `roles` names the parts the arrangement wants and the registry each is looked up in
-    ("norm", "mixer", "feed_forward", ...: the keys of REGISTRIES).  The decoder builds them and
-    hands them over as a dict; `caches` and `states` in `forward` are dicts by role that hold an
-    entry for every part that declared a cache or a state."""
+    ("norm", "mixer", "feed_forward", ...: the keys of REGISTRIES); roles listed in `optional`
+    may be left out of a layer.  The decoder builds them and hands them over as a dict; `caches`
+    and `states` in `forward` are dicts by role that hold an entry for every part that declared a
+    cache or a state."""
 
     roles: Dict[str, str] = {}
+    optional: Tuple[str, ...] = ()
 
     def __init__(self, parts: Dict[str, Part]):
-        missing = [r for r in self.roles if r not in parts]
+        missing = [r for r in self.roles if r not in parts and r not in self.optional]
         extra = [r for r in parts if r not in self.roles]
         if missing or extra:
             raise ValueError(f"{type(self).__name__} takes the parts {sorted(self.roles)}; "
@@ -247,12 +253,13 @@ NORMS = Registry("norm")
 MIXERS = Registry("mixer")
 FEED_FORWARDS = Registry("feed-forward")
 POSITION_ENCODINGS = Registry("position encoding")
+SCALES = Registry("channel scale")
 BLOCKS = Registry("block arrangement")
 
 
 # a block's roles and the model's own parts name their registry by these keys
 REGISTRIES = {"embedding": EMBEDDINGS, "head": HEADS, "norm": NORMS, "mixer": MIXERS,
-              "feed_forward": FEED_FORWARDS, "position_encoding": POSITION_ENCODINGS}
+              "feed_forward": FEED_FORWARDS, "position_encoding": POSITION_ENCODINGS, "scale": SCALES}
 
 
 def register_embedding(name, factory, **kw): EMBEDDINGS.register(name, factory, **kw)
@@ -261,4 +268,5 @@ def register_norm(name, factory, **kw): NORMS.register(name, factory, **kw)
 def register_mixer(name, factory, **kw): MIXERS.register(name, factory, **kw)
 def register_feed_forward(name, factory, **kw): FEED_FORWARDS.register(name, factory, **kw)
 def register_position_encoding(name, factory, **kw): POSITION_ENCODINGS.register(name, factory, **kw)
+def register_scale(name, factory, **kw): SCALES.register(name, factory, **kw)
 def register_block(name, factory, **kw): BLOCKS.register(name, factory, **kw)

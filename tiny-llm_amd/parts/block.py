@@ -1,7 +1,12 @@
 """Block arrangements.  "pre_norm" is Llama's: x + mixer(norm(x)), then
-x + ffn(norm(x)) (tiny_llm/parser/llama_parser.cpp:194-255)."""
+x + ffn(norm(x)) (tiny_llm/parser/llama_parser.cpp:194-255).  "output_norm" puts the norm on each
+sublayer's result instead: x + scale * norm(mixer(x)), then x + scale * norm(ffn(x)); the
+sublayers read the residual stream itself."""
 from __future__ import annotations
 
+import torch
+
+from ..kernels import ops
 from .base import Block, register_block
 
 
@@ -46,4 +51,58 @@ class PreNormBlock(Block):
         return norm.forward(x)
 
 
+class OutputNormBlock(Block):
+    """x <- x + s1 * norm1(mixer(x)); x <- x + s2 * norm2(ffn(x)).  The channel scales and the
+    feed-forward (with its norm and scale) may be left out.  The sublayers are called with
+    `residual=None` and return their result by itself in float32; norm, scale and the sum in float32
+    are one kernel, which also writes the copy of x in the engine's element type that the next
+    sublayer's products read (in float32 they read x itself)."""
+    roles = {"mixer": "mixer", "mixer_norm": "norm", "mixer_scale": "scale",
+             "ffn": "feed_forward", "ffn_norm": "norm", "ffn_scale": "scale"}
+    optional = ("mixer_scale", "ffn", "ffn_norm", "ffn_scale")
+
+    class _WantsCopy:
+        """What this arrangement shows as its `first_norm`: the block in front may hand over the
+        copy of x in the engine's element type instead of a prepared norm."""
+
+    def __init__(self, parts):
+        super().__init__(parts)
+        self.mixer, self.mixer_norm = parts["mixer"], parts["mixer_norm"]
+        self.mixer_scale = parts.get("mixer_scale")
+        self.ffn, self.ffn_norm, self.ffn_scale = parts.get("ffn"), parts.get("ffn_norm"), parts.get("ffn_scale")
+        if (self.ffn is None) != (self.ffn_norm is None) or (self.ffn is None and self.ffn_scale is not None):
+            raise ValueError("output_norm: a feed-forward comes with its norm, and a scale only with both")
+        for n in (self.mixer_norm, self.ffn_norm):
+            if n is not None and not hasattr(n, "add_normed"):
+                raise ValueError(f"output_norm: the norm {type(n).__name__} cannot sit on a sublayer's output (no add_normed)")
+        self.first_norm = self._WantsCopy()
+
+    def forward(self, x, ctx, caches, states):
+        return self.forward_chained(x, ctx, caches, states)[0]
+
+    def _input(self, x, name):
+        if x.dtype == self.mixer.dtype:
+            return x
+        return ops.cast_rows(x, ops.scratch(name, x.shape, self.mixer.dtype, x.device, rotate=2))
+
+    def forward_chained(self, x, ctx, caches, states, prepared=None, next_norm=None):
+        """`prepared`: the copy of x in the engine's element type, if the block in front was of this
+        kind; returned likewise for the block behind (`next_norm` is then its `first_norm`)."""
+        low = x.dtype != self.mixer.dtype          # the products read a copy in the engine's type
+        h = prepared if (low and isinstance(prepared, torch.Tensor)) else self._input(x, "stream_copy")
+        y = self.mixer.forward(h, ctx, caches.get("mixer"), states.get("mixer"), None)
+        want_after = low and (self.ffn is not None or isinstance(next_norm, self._WantsCopy))
+        copy = ops.scratch("stream_copy", x.shape, self.mixer.dtype, x.device, rotate=2) if want_after else None
+        self.mixer_norm.add_normed(y, x, self.mixer_scale.weight if self.mixer_scale is not None else None, copy)
+        if self.ffn is None:
+            return x, copy
+        y = self.ffn.forward(copy if low else x, ctx, None)
+        copy = None
+        if low and isinstance(next_norm, self._WantsCopy):
+            copy = ops.scratch("stream_copy", x.shape, self.mixer.dtype, x.device, rotate=2)
+        self.ffn_norm.add_normed(y, x, self.ffn_scale.weight if self.ffn_scale is not None else None, copy)
+        return x, copy
+
+
 register_block("pre_norm", PreNormBlock)
+register_block("output_norm", OutputNormBlock)

@@ -1,0 +1,129 @@
+"""The gated delta rule with a decay per head and key channel: a recurrent mixer.
+
+Per token (h is the mixer's input, [out, in] weights applied as W h):
+    q, k = silu(conv(W_q h)), silu(conv(W_k h))     kv_heads x dim, short causal convolution per channel
+    v    = silu(conv(W_v h))                         heads x vdim
+    q <- q / sqrt(|q|^2 + 1e-6) * dim^-1/2,  k <- k / sqrt(|k|^2 + 1e-6)       per head
+    beta = sigmoid(W_b h)                            per head
+    g    = exp(-exp(A_log) * softplus(W_a2 (W_a1 h) + dt_bias))                 heads x dim
+    per head:  S <- diag(g) S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
+    out  = W_o concat_heads( w_norm * unit_rms(o) * sigmoid(W_g2 (W_g1 h)) )
+Head n reads q/k head n // (heads / kv_heads).  Per request the part keeps S [heads, dim, vdim] and the
+last taps - 1 inputs of every convolution, in ONE float32 state row; the cache manager zeroes it when
+the request is admitted.  Everything that enters the recurrence is float32 in both precisions.
+
+The products: one reads h for [q | k | v | a1 | g1 | b] (segments start at multiples of 8 columns, the
+rows between are zero), one turns [a1 | g1] into [a | g] (a block-diagonal weight: one launch for
+the two low-rank products), one is W_o.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional
+
+import torch
+
+from ..kernels import ops
+from .base import Mixer, StateSpec, WeightSpec, register_mixer
+
+
+def _pad8(n: int) -> int:
+    return -(-n // 8) * 8
+
+
+class ChannelDelta(Mixer):
+    graph_safe = True
+
+    def __init__(self, prefix, dtype, device, *, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
+                 value_dim: int, conv_taps: int, decay_rank: int, gate_rank: int, eps: float,
+                 names: Dict[str, str] = None):
+        super().__init__(prefix, dtype, device)
+        self.hidden_size, self.num_heads, self.num_kv_heads = int(hidden_size), int(num_heads), int(num_kv_heads)
+        self.head_dim, self.value_dim, self.taps = int(head_dim), int(value_dim), int(conv_taps)
+        self.decay_rank, self.gate_rank, self.eps = int(decay_rank), int(gate_rank), float(eps)
+        ops.check_delta_sizes(self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim, self.taps)
+        if self.decay_rank <= 0 or self.gate_rank <= 0:
+            raise ValueError(f"{prefix}: the ranks of the decay's and the gate's projections must be positive")
+        ops.check_linear_sizes(dtype, self.hidden_size, f"{prefix}: hidden_size")
+        ops.check_linear_sizes(dtype, self.num_heads * self.value_dim, f"{prefix}: heads * value_dim")
+        H, KH, D, V = self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim
+        self.qk_size, self.v_size = KH * D, H * V
+        self.channels = 2 * self.qk_size + self.v_size
+        # columns of the product that reads h
+        self.low_off = _pad8(self.channels)
+        self.ra, self.rg = _pad8(self.decay_rank), _pad8(self.gate_rank)
+        self.b_off = self.low_off + self.ra + self.rg
+        self.in_width = self.b_off + _pad8(H)
+        self.state_size = H * D * V
+        n = {k: k for k in ("q", "k", "v", "b", "A_log", "norm", "a1", "a2", "dt_bias", "g1", "g2", "o")}
+        n.update({"q_conv": "q.conv", "k_conv": "k.conv", "v_conv": "v.conv"})
+        n.update(names or {})
+        self.names = {k: f"{prefix}.{v}" for k, v in n.items()}
+        self.w_in = self.w_low = self.w_o = None
+        self.conv_w = self.a_log = self.dt_bias = self.w_norm = None
+
+    # ---------------------------------------------------------------- declarations
+    def weights(self) -> List[WeightSpec]:
+        n, W, H, D, V = self.names, self.hidden_size, self.num_heads, self.head_dim, self.value_dim
+        vec = dict(role="vector")
+        return [WeightSpec(n["q"], (self.qk_size, W)), WeightSpec(n["q_conv"], (self.qk_size, self.taps), **vec),
+                WeightSpec(n["k"], (self.qk_size, W)), WeightSpec(n["k_conv"], (self.qk_size, self.taps), **vec),
+                WeightSpec(n["v"], (self.v_size, W)), WeightSpec(n["v_conv"], (self.v_size, self.taps), **vec),
+                WeightSpec(n["b"], (H, W)), WeightSpec(n["A_log"], (H,), **vec),
+                WeightSpec(n["norm"], (V,), role="vector", init="ones"),
+                WeightSpec(n["a1"], (self.decay_rank, W)), WeightSpec(n["a2"], (H * D, self.decay_rank)),
+                WeightSpec(n["dt_bias"], (H * D,), **vec),
+                WeightSpec(n["g1"], (self.gate_rank, W)), WeightSpec(n["g2"], (H * V, self.gate_rank)),
+                WeightSpec(n["o"], (W, H * V))]
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        n, H, D, V = self.names, self.num_heads, self.head_dim, self.value_dim
+        dev = tensors[n["q"]].device
+        w_in = torch.zeros((self.in_width, self.hidden_size), dtype=self.dtype, device=dev)
+        at = 0
+        for key in ("q", "k", "v"):
+            t = tensors[n[key]]
+            w_in[at:at + t.shape[0]] = t
+            at += t.shape[0]
+        w_in[self.low_off:self.low_off + self.decay_rank] = tensors[n["a1"]]
+        w_in[self.low_off + self.ra:self.low_off + self.ra + self.gate_rank] = tensors[n["g1"]]
+        w_in[self.b_off:self.b_off + H] = tensors[n["b"]]
+        self.w_in = w_in
+        w_low = torch.zeros((H * D + H * V, self.ra + self.rg), dtype=self.dtype, device=dev)
+        w_low[:H * D, :self.decay_rank] = tensors[n["a2"]]
+        w_low[H * D:, self.ra:self.ra + self.gate_rank] = tensors[n["g2"]]
+        self.w_low = w_low
+        self.w_o = tensors[n["o"]].contiguous()
+        f32 = lambda t: t.to(torch.float32).contiguous()
+        self.conv_w = torch.cat([f32(tensors[n[k]]) for k in ("q_conv", "k_conv", "v_conv")], dim=0).contiguous()
+        self.a_log, self.dt_bias, self.w_norm = f32(tensors[n["A_log"]]), f32(tensors[n["dt_bias"]]), f32(tensors[n["norm"]])
+
+    def state_spec(self) -> StateSpec:
+        return StateSpec((self.state_size + self.channels * (self.taps - 1),), torch.float32)
+
+    # --------------------------------------------------------------------- compute
+    def forward(self, h, ctx, cache, state, residual):
+        T, dev = h.shape[0], h.device
+        H, KH, D, V = self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim
+        p = ops.scratch("delta_in", (T, self.in_width), self.dtype, dev)
+        ops.linear(h, self.w_in, p)
+        low = ops.scratch("delta_low", (T, H * D + H * V), torch.float32, dev)
+        ops.linear(p[:, self.low_off:self.low_off + self.ra + self.rg], self.w_low, low)
+        qn = ops.scratch("delta_q", (T * H * D,), torch.float32, dev)
+        kn = ops.scratch("delta_k", (T * H * D,), torch.float32, dev)
+        dec = ops.scratch("delta_decay", (T * H * D,), torch.float32, dev)
+        vc = ops.scratch("delta_v", (T * H * V,), torch.float32, dev)
+        beta = ops.scratch("delta_beta", (T * H,), torch.float32, dev)
+        ops.delta_prepare(p, 0, self.b_off, low, self.conv_w, self.a_log, self.dt_bias, state, self.state_size,
+                          ctx.req_of_token, ctx.cu_seqlens_q, ctx.state_slots, qn, kn, vc, beta, dec, H, KH, D, V,
+                          self.taps, D ** -0.5)
+        ops.conv_state_update(p, 0, self.channels, state, self.state_size, ctx.cu_seqlens_q, ctx.state_slots, self.taps)
+        o = ops.scratch("delta_o", (T * H * V,), torch.float32, dev)
+        ops.delta_recurrence(qn, kn, vc, beta, dec, state, ctx.cu_seqlens_q, ctx.state_slots, o, H, D, V)
+        z = ops.scratch("delta_gated", (T, H * V), self.dtype, dev)
+        ops.head_norm_gate(o, self.w_norm, low[:, H * D:], z, H, V, self.eps)
+        if residual is None:
+            return ops.linear(z, self.w_o, ops.scratch("sublayer_out", (T, self.hidden_size), torch.float32, dev))
+        return ops.linear(z, self.w_o, residual, residual)
+
+
+register_mixer("channel_delta", ChannelDelta)

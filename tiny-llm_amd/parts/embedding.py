@@ -16,16 +16,17 @@ from .norm import LazyNorm
 class TokenEmbedding(Embedding):
     graph_safe = True
 
-    def __init__(self, prefix, dtype, device, *, vocab_size: int, hidden_size: int):
+    def __init__(self, prefix, dtype, device, *, vocab_size: int, hidden_size: int, weight_name: str = "weight"):
         super().__init__(prefix, dtype, device)
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
+        self.tensor_name = f"{prefix}.{weight_name}" if weight_name else prefix
         self.weight: Optional[torch.Tensor] = None
 
     def weights(self) -> List[WeightSpec]:
-        return [WeightSpec(f"{self.prefix}.weight", (self.vocab_size, self.hidden_size))]
+        return [WeightSpec(self.tensor_name, (self.vocab_size, self.hidden_size))]
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
-        self.weight = tensors[f"{self.prefix}.weight"].contiguous()
+        self.weight = tensors[self.tensor_name].contiguous()
 
     def forward(self, tokens: torch.Tensor, ctx=None) -> torch.Tensor:
         out = ops.scratch("residual", (tokens.numel(), self.hidden_size), torch.float32, tokens.device)
@@ -36,27 +37,35 @@ class LMHead(Head):
     graph_safe = True
     accepts_lazy_norm = True
 
-    def __init__(self, prefix, dtype, device, *, vocab_size: int, hidden_size: int, tied_to: str = None):
+    def __init__(self, prefix, dtype, device, *, vocab_size: int, hidden_size: int, tied_to: str = None,
+                 weight_name: str = "weight", softcap: float = 0.0):
+        """softcap c > 0: logits <- c * tanh(logits / c)."""
         super().__init__(prefix, dtype, device)
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
         self.tied_to = tied_to          # weight prefix of the embedding whose table this head shares
+        self.tensor_name = f"{prefix}.{weight_name}" if weight_name else prefix
+        self.softcap = float(softcap or 0.0)
+        if self.softcap < 0:
+            raise ValueError("the soft cap of the logits must be positive (0: none)")
         ops.check_linear_sizes(dtype, self.hidden_size, f"{prefix}: hidden_size")
         self.weight: Optional[torch.Tensor] = None
 
     def weights(self) -> List[WeightSpec]:
         alias = f"{self.tied_to}.weight" if self.tied_to else None
-        return [WeightSpec(f"{self.prefix}.weight", (self.vocab_size, self.hidden_size), alias_of=alias)]
+        return [WeightSpec(self.tensor_name, (self.vocab_size, self.hidden_size), alias_of=alias)]
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
-        self.weight = tensors[f"{self.prefix}.weight"].contiguous()
+        self.weight = tensors[self.tensor_name].contiguous()
 
     def forward(self, h) -> torch.Tensor:
         """h: activations [n, H], or a LazyNorm whose norm rides in the product."""
         if isinstance(h, LazyNorm):
             out = torch.empty((h.num_rows, self.vocab_size), dtype=torch.float32, device=h.x.device)
-            return h.linear(self.weight, out)
-        out = torch.empty((h.shape[0], self.vocab_size), dtype=torch.float32, device=h.device)
-        return ops.linear(h, self.weight, out)
+            out = h.linear(self.weight, out)
+        else:
+            out = torch.empty((h.shape[0], self.vocab_size), dtype=torch.float32, device=h.device)
+            out = ops.linear(h, self.weight, out)
+        return ops.softcap(out, self.softcap) if self.softcap else out
 
 
 register_embedding("token_embedding", TokenEmbedding)

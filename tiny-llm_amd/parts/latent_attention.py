@@ -1,0 +1,153 @@
+"""Causal attention whose cache holds one latent vector per token instead of keys and values.
+
+Per token (h is the mixer's input, [out, in] weights applied as W h):
+    c_q = w_dqn * unit_rms(W_dq h)                 q = W_uq c_q, per head [dim unrotated | rot_dim rotated]
+    [c_raw | kr_raw] = W_dkv h                     c = w_dkvn * unit_rms(c_raw), kr = rotate(kr_raw)
+    head n:  k_n = [W_uk,n c | kr],  v_n = W_uv,n c
+    score = (q_unrotated . W_uk,n c + rotate(q_rotated) . kr) * scale, softmax over positions j <= i
+    out = W_o concat_n( sigmoid(W_g h)_n * sum_j p_j v_j )
+Only c and kr are cached (pages [block, kv_rank] and [block, rot_dim]).  A layer built with
+`shares_cache=True` has no W_dkv: the plan lets it read the cache of an earlier layer, with its own
+W_uk, W_uv and queries.
+
+The up projections never touch the cache: q' = W_uk,n^T q_unrotated is formed per query
+([T, heads, kv_rank], float32), the kernel scores [q' | q_rotated] against [c | kr] and returns
+sum_j p_j c_j, and W_uv,n is applied to that.  The cache is read once per head as it lies, whatever
+the cut of the prompt; nothing of the context is projected again when a portion arrives.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional
+
+import torch
+
+from ..kernels import ops
+from .base import CacheSpec, CacheTensor, LayerCache, Mixer, POSITION_ENCODINGS, WeightSpec, register_mixer
+
+
+def _pad8(n: int) -> int:
+    return -(-n // 8) * 8
+
+
+class LatentAttention(Mixer):
+    graph_safe = True
+
+    def __init__(self, prefix, dtype, device, *, hidden_size: int, num_heads: int, head_dim: int, rot_dim: int,
+                 value_dim: int, q_rank: int, kv_rank: int, scale: float, eps: float, position: dict = None,
+                 shares_cache: bool = False, gated: bool = True, names: Dict[str, str] = None):
+        """head_dim: unrotated query/key dims per head; rot_dim: rotated dims behind them (the position
+        encoding rotates its first `rotary_dim`); scale: the factor of the scores, as given."""
+        super().__init__(prefix, dtype, device)
+        self.hidden_size, self.num_heads = int(hidden_size), int(num_heads)
+        self.head_dim, self.rot_dim, self.value_dim = int(head_dim), int(rot_dim), int(value_dim)
+        self.q_rank, self.kv_rank = int(q_rank), int(kv_rank)
+        self.scale, self.eps = float(scale), float(eps)
+        self.shares_cache, self.gated = bool(shares_cache), bool(gated)
+        if min(self.num_heads, self.head_dim, self.value_dim, self.q_rank, self.kv_rank) <= 0:
+            raise ValueError(f"{prefix}: heads, head sizes and ranks must be positive")
+        ops.check_latent_sizes(self.kv_rank, self.rot_dim)
+        for n, what in ((self.hidden_size, "hidden_size"), (self.q_rank, "q_rank"), (self.kv_rank, "kv_rank"),
+                        (self.head_dim, "head_dim"), (self.head_dim + self.rot_dim, "head_dim + rot_dim"),
+                        (self.num_heads * self.value_dim, "heads * value_dim"), (self.value_dim, "value_dim")):
+            ops.check_linear_sizes(dtype, n, f"{prefix}: {what}")
+        pos = dict(position or {"kind": "none"})
+        kind = pos.pop("kind")
+        self.position = POSITION_ENCODINGS.get(kind)(f"{prefix}.position", dtype, device, **pos)
+        tables = self.position.rotary_tables()
+        if (tables is None) != (self.rot_dim == 0) or getattr(self.position, "pairing", "half") != "half":
+            raise ValueError(f"{prefix}: rot_dim dims need a rotary encoding that pairs (i, i + dims/2)")
+        self.rdims = tables[2] if tables is not None else 0
+        if self.rdims > self.rot_dim:
+            raise ValueError(f"{prefix}: the encoding rotates {self.rdims} dims, the head has {self.rot_dim} for it")
+        n = {"dq": "dq", "dq_norm": "dq.norm", "uq": "uq", "dkv": "dkv", "dkv_norm": "dkv.norm", "uk": "uk",
+             "uv": "uv", "g": "g", "o": "o"}
+        n.update(names or {})
+        self.names = {k: f"{prefix}.{v}" for k, v in n.items()}
+        # columns of the one product that reads h: [query latent | latent and key part | gate], each
+        # starting at a multiple of 8 (the rows between are zero)
+        self.q_off = 0
+        self.kv_off = _pad8(self.q_rank)
+        self.g_off = self.kv_off + (0 if self.shares_cache else _pad8(self.kv_rank + self.rot_dim))
+        self.down_width = self.g_off + (_pad8(self.num_heads) if self.gated else 0)
+        self.w_down = self.w_uq = self.w_uk_t = self.w_uv = self.w_o = None
+        self.w_dq_norm = self.w_dkv_norm = None
+
+    # ---------------------------------------------------------------- declarations
+    def weights(self) -> List[WeightSpec]:
+        n, W, H = self.names, self.hidden_size, self.num_heads
+        out = [WeightSpec(n["dq"], (self.q_rank, W)), WeightSpec(n["dq_norm"], (self.q_rank,), role="vector", init="ones"),
+               WeightSpec(n["uq"], (H * (self.head_dim + self.rot_dim), self.q_rank))]
+        if not self.shares_cache:
+            out += [WeightSpec(n["dkv"], (self.kv_rank + self.rot_dim, W)),
+                    WeightSpec(n["dkv_norm"], (self.kv_rank,), role="vector", init="ones")]
+        out += [WeightSpec(n["uk"], (H * self.head_dim, self.kv_rank)),
+                WeightSpec(n["uv"], (H * self.value_dim, self.kv_rank))]
+        if self.gated:
+            out.append(WeightSpec(n["g"], (H, W)))
+        out.append(WeightSpec(n["o"], (W, H * self.value_dim)))
+        return out
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        n, H = self.names, self.num_heads
+        down = torch.zeros((self.down_width, self.hidden_size), dtype=self.dtype, device=tensors[n["dq"]].device)
+        down[:self.q_rank] = tensors[n["dq"]]
+        if not self.shares_cache:
+            down[self.kv_off:self.kv_off + self.kv_rank + self.rot_dim] = tensors[n["dkv"]]
+            self.w_dkv_norm = tensors[n["dkv_norm"]].to(torch.float32).contiguous()
+        if self.gated:
+            down[self.g_off:self.g_off + H] = tensors[n["g"]]
+        self.w_down = down
+        self.w_dq_norm = tensors[n["dq_norm"]].to(torch.float32).contiguous()
+        self.w_uq = tensors[n["uq"]].contiguous()
+        # per head the transpose of W_uk: q' = W_uk^T q is a product with [kv_rank, head_dim] weights
+        self.w_uk_t = tensors[n["uk"]].view(H, self.head_dim, self.kv_rank).transpose(1, 2).contiguous()
+        self.w_uv = tensors[n["uv"]].contiguous()
+        self.w_o = tensors[n["o"]].contiguous()
+
+    def cache_spec(self) -> CacheSpec:
+        tensors = [CacheTensor("latent", (self.kv_rank,), 0)]
+        if self.rot_dim:
+            tensors.append(CacheTensor("rope_key", (self.rot_dim,), 0))
+        return CacheSpec(tuple(tensors), "full", 0)
+
+    # --------------------------------------------------------------------- compute
+    def forward(self, h, ctx, cache: LayerCache, state, residual):
+        if cache.write == self.shares_cache:
+            raise ValueError(f"{self.prefix}: a layer with a down projection of its own writes its cache, "
+                             "one without reads another layer's")
+        T, dev, H = h.shape[0], h.device, self.num_heads
+        R, D, V, KR = self.rot_dim, self.head_dim, self.value_dim, self.kv_rank
+        tables = self.position.rotary_tables()
+        cos, sin = (tables[0], tables[1]) if tables is not None else (None, None)
+        latent, rope = cache.tensors["latent"], cache.tensors.get("rope_key")
+        down = ops.scratch("latent_down", (T, self.down_width), self.dtype, dev)
+        ops.linear(h, self.w_down, down)
+        cq = ops.scratch("latent_cq", (T, self.q_rank), self.dtype, dev)
+        if self.shares_cache:
+            ops.latent_prepare(down, self.q_off, self.q_rank, self.w_dq_norm, self.eps, cq)
+        else:
+            ops.latent_prepare(down, self.q_off, self.q_rank, self.w_dq_norm, self.eps, cq, self.kv_off, KR, R,
+                               self.rdims, self.w_dkv_norm, ctx.positions, cos, sin, ctx.slot_mappings[cache.group],
+                               latent, rope)
+        q = ops.scratch("latent_q", (T, H * (D + R)), self.dtype, dev)
+        ops.linear(cq, self.w_uq, q)
+        # [W_uk^T q_unrotated | rotate(q_rotated)] per head, float32
+        qa = ops.scratch("latent_qa", (T, H, KR + R), torch.float32, dev)
+        q3, qa2 = q.view(T, H, D + R), qa.view(T, H * (KR + R))
+        for n in range(H):
+            ops.linear(q3[:, n, :D], self.w_uk_t[n], qa2[:, n * (KR + R):n * (KR + R) + KR])
+        if R:
+            ops.rotate_into(q, H, D + R, D, R, self.rdims, ctx.positions, cos, sin, qa, KR)
+        mix = ops.scratch("latent_mix", (T, H, KR), self.dtype, dev)
+        gate = down[:, self.g_off:self.g_off + H] if self.gated else None
+        ops.latent_attention(qa, latent, rope, ctx.block_tables[cache.group], ctx.req_of_token, ctx.positions, mix,
+                             self.scale, gate)
+        o = ops.scratch("latent_heads", (T, H * V), self.dtype, dev)
+        for n in range(H):
+            ops.linear(mix[:, n, :], self.w_uv[n * V:(n + 1) * V], o[:, n * V:(n + 1) * V])
+        if residual is None:
+            return ops.linear(o, self.w_o, ops.scratch("sublayer_out", (T, self.hidden_size), torch.float32, dev))
+        return ops.linear(o, self.w_o, residual, residual)
+
+
+register_mixer("latent_attention", LatentAttention)

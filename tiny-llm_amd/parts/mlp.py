@@ -56,4 +56,49 @@ class SwiGLU(FeedForward):
         return out if next_norm is None else (out, prepared)
 
 
+class ClampedGLU(FeedForward):
+    """down(g * sigmoid(alpha * g) * (u + shift)) with g = min(gate(h), limit) and
+    u = clamp(up(h), -limit, limit).  Gate and up weights are stacked on load into one [2F, H]
+    matrix (one product); the activation runs on its result in the engine's element type.
+
+    `names`: the tensors' names below the prefix, (gate, up, down).  With `residual=None` the
+    result is returned by itself in float32 (a block that norms the sublayer's output adds it)."""
+    graph_safe = True
+
+    def __init__(self, prefix, dtype, device, *, hidden_size: int, intermediate_size: int, limit: float,
+                 alpha: float = 1.702, shift: float = 1.0, names=("gate", "up", "down")):
+        super().__init__(prefix, dtype, device)
+        self.hidden_size = int(hidden_size)
+        self.intermediate_size = int(intermediate_size)
+        self.limit, self.alpha, self.shift = float(limit), float(alpha), float(shift)
+        if not self.limit > 0:
+            raise ValueError(f"{prefix}: the limit of the gated unit must be positive")
+        ops.check_linear_sizes(dtype, self.hidden_size, f"{prefix}: hidden_size")
+        ops.check_linear_sizes(dtype, self.intermediate_size, f"{prefix}: intermediate_size")
+        self.names = tuple(f"{prefix}.{n}" for n in names)
+        self.w_gate_up: Optional[torch.Tensor] = None
+        self.w_down: Optional[torch.Tensor] = None
+
+    def weights(self) -> List[WeightSpec]:
+        H, I = self.hidden_size, self.intermediate_size
+        gate, up, down = self.names
+        return [WeightSpec(gate, (I, H)), WeightSpec(up, (I, H)), WeightSpec(down, (H, I))]
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        gate, up, down = self.names
+        self.w_gate_up = torch.cat([tensors[gate], tensors[up]], dim=0).contiguous()
+        self.w_down = tensors[down].contiguous()
+
+    def forward(self, h, ctx, residual):
+        T, dev = h.shape[0], h.device
+        gu = ops.scratch("ffn_gate_up", (T, 2 * self.intermediate_size), self.dtype, dev)
+        ops.linear(h, self.w_gate_up, gu)
+        z = ops.scratch("ffn_gated", (T, self.intermediate_size), self.dtype, dev)
+        ops.clamped_glu(gu, z, self.limit, self.alpha, self.shift)
+        if residual is None:
+            return ops.linear(z, self.w_down, ops.scratch("sublayer_out", (T, self.hidden_size), torch.float32, dev))
+        return ops.linear(z, self.w_down, residual, residual)
+
+
 register_feed_forward("swiglu", SwiGLU)
+register_feed_forward("clamped_glu", ClampedGLU)

@@ -11,7 +11,7 @@ from typing import Dict, List, Optional
 import torch
 
 from ..kernels import ops
-from .base import Norm, WeightSpec, register_norm
+from .base import ChannelScale, Norm, WeightSpec, register_norm, register_scale
 
 
 class LazyNorm:
@@ -58,18 +58,33 @@ class RMSNorm(Norm):
     graph_safe = True
     F32_FUSED_ROWS = 16      # measured on whole steps: beyond, the norm's own kernel is as fast or faster
 
-    def __init__(self, prefix, dtype, device, *, hidden_size: int, eps: float, init: str = "ones"):
+    def __init__(self, prefix, dtype, device, *, hidden_size: int, eps: float, init: str = "ones",
+                 offset: float = 0.0, weight_name: str = "weight"):
+        """offset: the effective weight is offset + the stored one (1.0 for checkpoints that store
+        the weight around zero); it is then kept in float32.  weight_name: the tensor's name below
+        the prefix ("" if the prefix itself names it)."""
         super().__init__(prefix, dtype, device)
         self.hidden_size = int(hidden_size)
         self.eps = float(eps)
-        self.init = init
+        self.offset = float(offset)
+        self.init = init if not self.offset else "zeros"
+        self.tensor_name = f"{prefix}.{weight_name}" if weight_name else prefix
         self.weight: Optional[torch.Tensor] = None
 
     def weights(self) -> List[WeightSpec]:
-        return [WeightSpec(f"{self.prefix}.weight", (self.hidden_size,), role="vector", init=self.init)]
+        return [WeightSpec(self.tensor_name, (self.hidden_size,), role="vector", init=self.init)]
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
-        self.weight = tensors[f"{self.prefix}.weight"].contiguous()
+        w = tensors[self.tensor_name]
+        # offset + w is formed in float32: in bfloat16 the sum would lose what the stored weight says
+        self.weight = (w.to(torch.float32) + self.offset).contiguous() if self.offset else w.contiguous()
+
+    def add_normed(self, y: torch.Tensor, x: torch.Tensor, scale: Optional[torch.Tensor] = None,
+                   copy: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """x += scale * norm(y) for a norm that sits on a sublayer's output (y float32, one kernel);
+        `copy` receives the new x in its own element type."""
+        w = self.weight if self.weight.dtype == torch.float32 else self.weight.to(torch.float32)
+        return ops.norm_scale_add(y, w, self.eps, x, scale, copy)
 
     def lazy(self, x: torch.Tensor, rows: Optional[torch.Tensor] = None, prepared=None):
         """The norm rides in the consumer's first product: in bfloat16 always (`ops.linear_norm`), in
@@ -100,4 +115,22 @@ class RMSNorm(Norm):
         return ops.rmsnorm(x, self.weight, self.eps, out, rows)
 
 
+class VectorScale(ChannelScale):
+    """A learned vector that multiplies a sublayer's result channel by channel; kept in float32.
+    The tensor is named by the prefix itself."""
+    graph_safe = True
+
+    def __init__(self, prefix, dtype, device, *, hidden_size: int):
+        super().__init__(prefix, dtype, device)
+        self.hidden_size = int(hidden_size)
+        self.weight: Optional[torch.Tensor] = None
+
+    def weights(self) -> List[WeightSpec]:
+        return [WeightSpec(self.prefix, (self.hidden_size,), role="vector", init="ones")]
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        self.weight = tensors[self.prefix].to(torch.float32).contiguous()
+
+
 register_norm("rmsnorm", RMSNorm)
+register_scale("vector", VectorScale)

@@ -286,6 +286,8 @@ def _scale_and_shift(spec: WeightSpec, std: float, norm_std: float) -> Tuple[flo
     """value = shift + scale * z for this tensor."""
     if spec.init in ("ones", "around_one"):
         return float(norm_std), 1.0
+    if spec.init in ("zeros", "around_zero"):        # weights stored as a distance from one
+        return float(norm_std), 0.0
     return float(std), 0.0
 
 
