@@ -13,7 +13,8 @@ Llama-3-8B shape; 64 requests of 1,024 tokens that nearly fill the cache at the 
 `--only` picks a part (for profiling), or one of the measurements that are not part of the line:
 `attention` (the attention kernels alone at contexts up to 131,072 tokens), `long_context` (the Llama-3-8B
 shape with 8 requests of 32,000 tokens and one of 131,000), `decode_shapes` (decode steps at the two larger
-shapes by batch), `host` (a step's wall time against its time on the GPU).
+shapes by batch), `host` (a step's wall time against its time on the GPU), `lufazen` (the Lufazen design,
+recurrent and latent-attention layers, at two sizes beside a Llama of equal size: prefill, decode, time by kernel).
 """
 import argparse
 import json
@@ -136,7 +137,7 @@ class Bench:
         from tiny_llm_amd import Engine
         self.torch = torch
         self.cfg, self.dtype = cfg, dtype
-        self.V = cfg["vocab_size"]
+        self.V = cfg.get("vocab_size") or cfg["vocab"]
         blocks = (max_batch * (prompt_len + total_new) + extra_tokens) // block_size + max_batch + 8
         if max_cache_tokens is not None:
             blocks = max_cache_tokens // block_size
@@ -695,7 +696,118 @@ def attention_sweep():
     return rows
 
 
+# ------------------------------------------------- the Lufazen design beside a Llama of equal size
+def lufazen_config(layers, width, ff, heads, vocab=32000):
+    """Layers in the order delta, delta, delta, attention (the second attention layer of a model reads
+    the first one's cache): heads of 128 key channels and 128 values in the recurrent layers; 128
+    unrotated + 64 rotated query/key dims, values of 128, latents of 512 (keys/values) and 768 (queries)
+    in the attention layers."""
+    out, first = [], None
+    for i in range(layers):
+        mlp = {"kind": "dense", "ff": ff, "limit": 7.0}
+        if i % 4 == 3:
+            m = {"heads": heads, "dim": 128, "rot_dim": 64, "vdim": 128, "q_rank": 768, "kv_rank": 512,
+                 "scale": 192 ** -0.5, "rot": {"base": 10000.0, "dims": 64,
+                                               "scaling": {"factor": 40.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}
+            if first is None:
+                first = i
+            elif (i // 4) % 2 == 1:
+                m["kv_from"] = first
+            out.append({"type": "latent_attention", "mixer": m, "mlp": mlp})
+        else:
+            out.append({"type": "channel_delta", "mlp": mlp,
+                        "mixer": {"heads": heads, "kv_heads": heads, "dim": 128, "vdim": 128, "conv": 4,
+                                  "decay_rank": 64, "gate_rank": 64}})
+    return {"architecture": "Lufazen", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "logit_softcap": 30.0,
+            "layers": out, "max_position": 8192}
+
+
+def kernels_by_name(run):
+    """Microseconds per step by kernel (the name up to its template arguments), from torch's profiler
+    around `run`; steps are counted by their embedding kernels."""
+    import torch
+    from torch.autograd import DeviceType
+    from torch.profiler import ProfilerActivity, profile
+    with profile(activities=[ProfilerActivity.CUDA]) as prof:
+        run()
+        torch.cuda.synchronize()
+    evs = [e for e in prof.events() if e.device_type == DeviceType.CUDA and "emcpy" not in e.name and "emset" not in e.name]
+    steps = max(1, sum(1 for e in evs if "embedding_kernel" in e.name))
+    out = {}
+    for e in evs:
+        name = e.name.split("<")[0].split("(")[0].replace("(anonymous namespace)::", "").replace("void ", "").strip()
+        t, n = out.get(name, (0.0, 0))
+        out[name] = (t + (e.time_range.end - e.time_range.start), n + 1)
+    return {k: {"us": round(t / steps, 1), "launches": round(n / steps, 1)} for k, (t, n) in sorted(out.items(), key=lambda kv: -kv[1][0])}
+
+
+def lufazen_figures(args):
+    """Prefill (2,048 tokens, whole) and decode (batches 1 and 8 behind 512-token prompts) of the
+    Lufazen design at two sizes, each beside a Llama with the same number of layers, width, feed-forward
+    size, heads of 128 and vocabulary; time by kernel for both; and for the kernels that only the new
+    design has, what the published peaks would allow (bytes over 8 TB/s or flops over the matrix peak)."""
+    import torch
+    dtype = args.dtype
+    out = {}
+    for name, (layers, width, ff, heads) in {"w2048": (8, 2048, 5632, 16), "w4096": (8, 4096, 14336, 32)}.items():
+        if args.layers:
+            layers = args.layers
+        row = {"layers": layers, "width": width, "ff": ff, "heads": heads}
+        for which, cfg in (("lufazen", lufazen_config(layers, width, ff, heads)),
+                           ("llama", llama(layers, width, heads, heads, ff, 32000, 10000.0, 8192))):
+            b = Bench(cfg, dtype, max_batch=8, total_new=args.steps + args.warmup + 200, block_size=args.block_size)
+            r = {}
+            t = b.prefill(3)
+            r["prefill_2048"] = {"ms": round(t * 1e3, 3), "tok_s": round(PREFILL_TOKENS / t, 1)}
+            for batch in (1, 8):
+                dt, _ = b.decode(batch, args.steps, args.warmup)
+                r[f"decode_b{batch}"] = {"ms_per_step": round(dt / args.steps * 1e3, 4), "tok_s": round(batch * args.steps / dt, 1)}
+            eng = b.engine
+            from tiny_llm_amd import SamplingParams
+
+            def one_prefill(seed):
+                rid = eng.add_request(gen_tokens(PREFILL_TOKENS, b.V, seed), SamplingParams.greedy(1, ignore_eos=True))
+                while eng.requests[rid].status != "finished":
+                    eng.step()
+            r["prefill_kernels"] = kernels_by_name(lambda: one_prefill(93))
+            ids = [eng.add_request(gen_tokens(PROMPT_LEN, b.V, 1000 + i), SamplingParams.greedy(200, ignore_eos=True)) for i in range(8)]
+            while any(eng.requests[i].num_computed < PROMPT_LEN for i in ids):
+                eng.step()
+            for _ in range(3):
+                eng.step()
+
+            def some_decode():
+                at = eng.steps_run
+                while eng.steps_run - at < 32:
+                    eng.step(max_decode_steps=32 - (eng.steps_run - at))
+            r["decode_b8_kernels"] = kernels_by_name(some_decode)
+            for i in ids:
+                eng.abort(i)
+            b.close()
+            row[which] = r
+        # what the peaks allow for the new design's own kernels, per layer of that kind
+        e = ELT[dtype]
+        T, ctx, B = PREFILL_TOKENS, PROMPT_LEN, 8
+        kr, rot = 512, 64
+        row["bounds_us"] = {
+            "latent_attention prefill (flops of scores and values over the latent, causal)":
+                round(2.0 * heads * (T * T / 2) * (2 * kr + rot) / (PEAK_TFLOPS[dtype] * 1e12) * 1e6, 1),
+            "latent_attention decode b8 (the cached latents once)":
+                round(B * ctx * (kr + rot) * e / (HBM_GBS * 1e9) * 1e6, 2),
+            "delta_recurrence decode b8 (the states read and written)":
+                round(2.0 * B * heads * 128 * 128 * 4 / (HBM_GBS * 1e9) * 1e6, 2),
+            "delta_recurrence prefill (6 flops per state element and token, float32 vector units at 157 TFLOP/s)":
+                round(6.0 * T * heads * 128 * 128 / (157.3e12) * 1e6, 1),
+        }
+        out[name] = row
+        print(json.dumps({name: row}), file=sys.stderr, flush=True)
+    return out
+
+
 def run(args):
+    if args.only == "lufazen":
+        print(json.dumps({"lufazen_beside_llama": lufazen_figures(args)}), flush=True)
+        return
     if args.only == "attention":
         print(json.dumps({"decode_attention": attention_sweep()}), flush=True)
         return
@@ -771,13 +883,14 @@ def main():
     ap.add_argument("--block-size", type=int, default=16)
     ap.add_argument("--only", default="all",
                     choices=["all", "headline", "decode", "prefill", "fp32", "kernels", "peaks", "llama3_8b", "llama3_8b_prefill", "llama2_13b", "host",
-                             "attention", "long_context", "decode_shapes"],
+                             "attention", "long_context", "decode_shapes", "lufazen"],
                     help="all: everything in one line; headline: the bfloat16 TinyLlama figures only; decode / prefill: "
                          "one of them (profiling); fp32: the float32 figures as the headline; kernels: decode with the time of "
                          "a step by kernel (torch's profiler); peaks / llama3_8b / "
                          "llama2_13b: that part alone; host: a step's wall time against its time on the GPU; attention: the "
                          "attention kernels alone at contexts up to 131,072 tokens; long_context: the Llama-3-8B shape with "
-                         "8 requests of 32,000 tokens and one of 131,000; decode_shapes: decode steps at the two larger shapes by batch")
+                         "8 requests of 32,000 tokens and one of 131,000; decode_shapes: decode steps at the two larger shapes by batch; "
+                         "lufazen: prefill and decode of the Lufazen design at two sizes beside a Llama of equal size, by kernel")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         if int(os.environ.get("RANK", "0")) == 0:

@@ -67,7 +67,10 @@ CONFIGS = {"A": (MIX_A, RANKS_A, 16), "B": (MIX_B, RANKS_B, 8), "latent": (ONLY_
 
 
 def random_weights(cfg, ranks, seed=0, sharpen=3.0):
-    """{name: float32 tensor}.  `ranks`: {layer: (rank of a1, rank of g1)} for the recurrent layers."""
+    """{name: float32 tensor}.  `ranks`: {layer: (rank of a1, rank of g1)} for the recurrent layers.
+    `sharpen`: the gain of the projections that make scores, gates and decays (3: far from uniform, a
+    misplaced key or a lost state moves the logits; 1: tame, so that bfloat16 rounding is not amplified)."""
+    lively = 2.0 if sharpen > 1.0 else 1.0
     rng = np.random.default_rng(seed)
     W, out = cfg["width"], {}
 
@@ -92,32 +95,32 @@ def random_weights(cfg, ranks, seed=0, sharpen=3.0):
                 vec(p + "mix.dkv.norm", m["kv_rank"], 1.0)
             mat(p + "mix.uk", H * D, m["kv_rank"])
             mat(p + "mix.uv", H * V, m["kv_rank"])
-            mat(p + "mix.g", H, W, gain=2.0)
+            mat(p + "mix.g", H, W, gain=lively)
             mat(p + "mix.o", W, H * V)
         else:
             H, KH, D, V, taps = m["heads"], m["kv_heads"], m["dim"], m["vdim"], m["conv"]
             ra, rg = ranks[i]
             for n, rows in (("q", KH * D), ("k", KH * D), ("v", H * V)):
-                mat(p + f"mix.{n}", rows, W, gain=2.0)
+                mat(p + f"mix.{n}", rows, W, gain=lively)
                 out[p + f"mix.{n}.conv"] = rng.standard_normal((rows, taps)) * 0.6
-            mat(p + "mix.b", H, W, gain=2.0)
+            mat(p + "mix.b", H, W, gain=lively)
             out[p + "mix.A_log"] = rng.uniform(-1.5, 0.5, H)
             vec(p + "mix.norm", V, 1.0)
             mat(p + "mix.a1", ra, W)
-            mat(p + "mix.a2", H * D, ra, gain=2.0)
+            mat(p + "mix.a2", H * D, ra, gain=lively)
             vec(p + "mix.dt_bias", H * D, -1.0, 1.0)
             mat(p + "mix.g1", rg, W)
-            mat(p + "mix.g2", H * V, rg, gain=2.0)
+            mat(p + "mix.g2", H * V, rg, gain=lively)
             mat(p + "mix.o", W, H * V)
         if l["mlp"] is not None:
             F = l["mlp"]["ff"]
-            mat(p + "mlp.gate", F, W, gain=2.0)
-            mat(p + "mlp.up", F, W, gain=2.0)
+            mat(p + "mlp.gate", F, W, gain=lively)
+            mat(p + "mlp.up", F, W, gain=lively)
             mat(p + "mlp.down", W, F)
             vec(p + "norm2", W)
             vec(p + "ls2", W, 0.7, 0.2)
     vec("final.norm", W)
-    mat("head", cfg["vocab"], W, gain=2.0)
+    mat("head", cfg["vocab"], W, gain=lively)
     return {k: torch.from_numpy(np.asarray(v, dtype=np.float32)) for k, v in out.items()}
 
 

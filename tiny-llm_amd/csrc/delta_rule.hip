@@ -171,6 +171,88 @@ __global__ __launch_bounds__(TL_WAVE) void head_norm_gate_kernel(const float* __
   for (int j = lane; j < vdim; j += TL_WAVE) dst[j] = from_f32<T>(src[j] * r * w[j] / (1.f + expf(-gp[j])));
 }
 
+// Sum over a workgroup of `nw` waves (nw <= 16); `red` is LDS of 16 floats.  Fixed order.
+__device__ __forceinline__ float block_sum_dyn(float v, float* red, int nw) {
+  v = wave_sum(v);
+  __syncthreads();
+  if (threadIdx.x % TL_WAVE == 0) red[threadIdx.x / TL_WAVE] = v;
+  __syncthreads();
+  float t = 0.f;
+  for (int i = 0; i < nw; ++i) t += red[i];
+  return t;
+}
+
+// A decode step in one kernel: every request brings ONE token.  One workgroup per (request, head),
+// a thread per value column: the convolutions, unit vectors, decay and beta of the token, the
+// recurrence on the column in registers, and the head's norm and gate on the way out
+// (z[t, h, :] = w * o / rms(o) * sigmoid(gate)).  The saved convolution inputs are read here and
+// brought up to date by conv_state_update_kernel behind it.
+template <typename T, int DIM>
+__global__ void delta_decode_kernel(
+    const T* __restrict__ p, int64_t p_stride, int conv_off, int b_off, const float* __restrict__ low, int64_t low_stride,
+    const float* __restrict__ conv_w, const float* __restrict__ a_log, const float* __restrict__ dt_bias,
+    const float* __restrict__ w_norm, float* __restrict__ state, int64_t state_stride, int64_t saved_off,
+    const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ state_slots, T* __restrict__ z, int heads,
+    int kv_heads, int dim, int vdim, int taps, float q_scale, float eps) {
+  __shared__ float qs[kMaxDim], ks[kMaxDim], gs[kMaxDim], red[16];
+  const int r = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+  const int nw = blockDim.x / TL_WAVE;
+  const int t = cu_seqlens[r];
+  if (cu_seqlens[r + 1] - t != 1) return;         // a padding request owns no state
+  const int kh = h / (heads / kv_heads);
+  float* row = state + (int64_t)state_slots[r] * state_stride;
+  const float* saved = row + saved_off;
+  const int q_ch = kh * dim, k_ch = kv_heads * dim + kh * dim, v_ch = 2 * kv_heads * dim + h * vdim;
+  float sq = 0.f, sk = 0.f;
+  const float rate = expf(a_log[h]);
+  for (int i = tid; i < dim; i += blockDim.x) {
+    const float q = conv_silu(p, p_stride, t, 0, conv_off + q_ch + i, saved + (int64_t)(q_ch + i) * (taps - 1),
+                              conv_w + (int64_t)(q_ch + i) * taps, taps);
+    const float k = conv_silu(p, p_stride, t, 0, conv_off + k_ch + i, saved + (int64_t)(k_ch + i) * (taps - 1),
+                              conv_w + (int64_t)(k_ch + i) * taps, taps);
+    qs[i] = q;
+    ks[i] = k;
+    sq += q * q;
+    sk += k * k;
+    gs[i] = expf(-rate * softplus(low[(int64_t)t * low_stride + h * dim + i] + dt_bias[h * dim + i]));
+  }
+  sq = block_sum_dyn(sq, red, nw);
+  sk = block_sum_dyn(sk, red, nw);      // its barriers also make qs, ks and gs visible
+  const float rq = q_scale / sqrtf(sq + 1e-6f), rk = 1.f / sqrtf(sk + 1e-6f);
+  const int col = tid;
+  float o = 0.f;
+  if (col < vdim) {
+    const float v = conv_silu(p, p_stride, t, 0, conv_off + v_ch + col, saved + (int64_t)(v_ch + col) * (taps - 1),
+                              conv_w + (int64_t)(v_ch + col) * taps, taps);
+    const float beta = 1.f / (1.f + expf(-to_f32(p[(int64_t)t * p_stride + b_off + h])));
+    float* S_mem = row + (int64_t)h * dim * vdim + col;
+    float S[DIM];
+#pragma unroll
+    for (int i = 0; i < DIM; ++i) S[i] = i < dim ? S_mem[(int64_t)i * vdim] : 0.f;
+    float acc = 0.f;
+#pragma unroll
+    for (int i = 0; i < DIM; ++i)
+      if (i < dim) {
+        S[i] *= gs[i];
+        acc = fmaf(S[i], ks[i] * rk, acc);
+      }
+    const float u = beta * (v - acc);
+#pragma unroll
+    for (int i = 0; i < DIM; ++i)
+      if (i < dim) {
+        S[i] = fmaf(ks[i] * rk, u, S[i]);
+        o = fmaf(S[i], qs[i] * rq, o);
+        S_mem[(int64_t)i * vdim] = S[i];
+      }
+  }
+  const float ss = block_sum_dyn(col < vdim ? o * o : 0.f, red, nw);
+  if (col < vdim) {
+    const float g = low[(int64_t)t * low_stride + heads * dim + h * vdim + col];
+    z[((int64_t)t * heads + h) * vdim + col] =
+        from_f32<T>(o / sqrtf(ss / (float)vdim + eps) * w_norm[col] / (1.f + expf(-g)));
+  }
+}
+
 }  // namespace
 
 #define TL_DISPATCH_T(dtype, ...)                 \
@@ -226,6 +308,35 @@ int tl_delta_recurrence(const float* qn, const float* kn, const float* vc, const
   else if (dim <= 128) TL_REC(128);
   else TL_REC(256);
 #undef TL_REC
+  return tl_launch_status();
+}
+
+// `low` row t: [decay pre-activations heads x dim | gate pre-activations heads x vdim], float32.
+int tl_delta_decode(const void* p, int64_t p_stride, int conv_off, int b_off, const float* low, int64_t low_stride,
+                    const float* conv_w, const float* a_log, const float* dt_bias, const float* w_norm, float* state,
+                    int64_t state_stride, int64_t saved_off, const int32_t* cu_seqlens, const int32_t* state_slots,
+                    void* z, int n_requests, int heads, int kv_heads, int dim, int vdim, int taps, float q_scale,
+                    float eps, int dtype, hipStream_t stream) {
+  if (n_requests <= 0) return TL_OK;
+  if (heads <= 0 || heads > 65535 || kv_heads <= 0 || heads % kv_heads || dim <= 0 || dim > kMaxDim || vdim <= 0 ||
+      vdim > 1024 || taps < 1 || taps > kMaxTaps)
+    return TL_ERR_ARG;
+  dim3 g(n_requests, heads), b((vdim + TL_WAVE - 1) / TL_WAVE * TL_WAVE);
+#define TL_DEC(TT, D)                                                                                               \
+  hipLaunchKernelGGL((delta_decode_kernel<TT, D>), g, b, 0, stream, (const TT*)p, p_stride, conv_off, b_off, low,   \
+                     low_stride, conv_w, a_log, dt_bias, w_norm, state, state_stride, saved_off, cu_seqlens,        \
+                     state_slots, (TT*)z, heads, kv_heads, dim, vdim, taps, q_scale, eps)
+#define TL_DEC_D(TT)                  \
+  if (dim <= 16) TL_DEC(TT, 16);      \
+  else if (dim <= 32) TL_DEC(TT, 32); \
+  else if (dim <= 64) TL_DEC(TT, 64); \
+  else if (dim <= 128) TL_DEC(TT, 128); \
+  else TL_DEC(TT, 256);
+  if (dtype == 0) { TL_DEC_D(float) }
+  else if (dtype == 1) { TL_DEC_D(bf16_t) }
+  else return TL_ERR_ARG;
+#undef TL_DEC_D
+#undef TL_DEC
   return tl_launch_status();
 }
 

@@ -152,6 +152,39 @@ __global__ __launch_bounds__(TL_WAVE) void latent_attention_kernel(
   }
 }
 
+// Small products per head for steps of few rows: out[t, h, n] = sum_k w[h, k, n] * in[t, h, k].
+// The weights lie [heads, inner, cols], so that the threads of a workgroup (one per output column)
+// read them in whole lines; a workgroup takes up to kRows rows at a time, whose inputs it keeps in LDS.
+constexpr int kRows = 8;
+constexpr int kMaxInner = 1024;
+template <typename TI, typename TW, typename TO>
+__global__ __launch_bounds__(kThreads) void head_products_kernel(const TI* __restrict__ in, int64_t in_stride,
+                                                                 int in_head_width, const TW* __restrict__ w,
+                                                                 TO* __restrict__ out, int64_t out_stride,
+                                                                 int out_head_width, int n_rows, int inner, int cols) {
+  __shared__ float xs[kRows][kMaxInner];
+  const int h = blockIdx.x, n = blockIdx.y * kThreads + threadIdx.x;
+  const int t0 = blockIdx.z * kRows, rows = min(kRows, n_rows - t0);
+  for (int e = threadIdx.x; e < rows * inner; e += kThreads) {
+    const int r = e / inner, k = e - r * inner;
+    xs[r][k] = to_f32(in[(int64_t)(t0 + r) * in_stride + (int64_t)h * in_head_width + k]);
+  }
+  __syncthreads();
+  if (n >= cols) return;
+  float acc[kRows];
+#pragma unroll
+  for (int r = 0; r < kRows; ++r) acc[r] = 0.f;
+  const TW* wp = w + (int64_t)h * inner * cols + n;
+  for (int k = 0; k < inner; ++k) {
+    const float wv = to_f32(wp[(int64_t)k * cols]);
+#pragma unroll
+    for (int r = 0; r < kRows; ++r) acc[r] = fmaf(wv, xs[r][k], acc[r]);      // rows beyond `rows` hold stale LDS: never stored
+  }
+#pragma unroll
+  for (int r = 0; r < kRows; ++r)
+    if (r < rows) out[(int64_t)(t0 + r) * out_stride + (int64_t)h * out_head_width + n] = from_f32<TO>(acc[r]);
+}
+
 }  // namespace
 
 #define TL_DISPATCH_T(dtype, ...)                 \
@@ -202,6 +235,27 @@ int tl_latent_attention(const float* qa, const void* latent, const void* rope, c
                                           (const T*)rope, block_tables, max_blocks, req_of_token, positions,
                                           (const T*)gate, gate_stride, (T*)out, heads, kv_rank, rot, block_size,
                                           scale);)
+  return tl_launch_status();
+}
+
+// in / out: rows with a stride, head h at column h * head_width.  w [heads, inner, cols] of in's type;
+// out float32 (out_dtype 0) or of in's type.
+int tl_head_products(const void* in, int64_t in_stride, int in_head_width, const void* w, void* out,
+                     int64_t out_stride, int out_head_width, int n_rows, int heads, int inner, int cols, int dtype,
+                     int out_dtype, hipStream_t stream) {
+  if (n_rows <= 0) return TL_OK;
+  if (heads <= 0 || inner <= 0 || inner > kMaxInner || cols <= 0 || inner > in_head_width || cols > out_head_width ||
+      (n_rows + kRows - 1) / kRows > 65535 || (cols + kThreads - 1) / kThreads > 65535)
+    return TL_ERR_ARG;
+  dim3 g(heads, (cols + kThreads - 1) / kThreads, (n_rows + kRows - 1) / kRows), b(kThreads);
+#define TL_HP(TI, TO)                                                                                              \
+  hipLaunchKernelGGL((head_products_kernel<TI, TI, TO>), g, b, 0, stream, (const TI*)in, in_stride, in_head_width, \
+                     (const TI*)w, (TO*)out, out_stride, out_head_width, n_rows, inner, cols)
+  if (dtype == 0 && out_dtype == 0) TL_HP(float, float);
+  else if (dtype == 1 && out_dtype == 0) TL_HP(bf16_t, float);
+  else if (dtype == 1 && out_dtype == 1) TL_HP(bf16_t, bf16_t);
+  else return TL_ERR_ARG;
+#undef TL_HP
   return tl_launch_status();
 }
 

@@ -1228,6 +1228,28 @@ def latent_attention(qa: torch.Tensor, latent: torch.Tensor, rope: Optional[torc
     return out
 
 
+HEAD_PRODUCT_ROWS = 32      # up to this many rows the per-head products of a step run as ONE launch
+HEAD_PRODUCT_INNER = 1024
+
+
+def head_products(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[t, h, :] = w[h]^T x[t, h, :] for every head in one launch (steps of few rows):
+    x [T, heads, >= inner] and out [T, heads, >= cols] may be views into wider rows (any row and
+    head stride, unit inner stride); w [heads, inner, cols] contiguous of x's type; out float32 or x's type."""
+    _dev(x, w, out)
+    T, H = x.shape[0], x.shape[1]
+    inner, cols = w.shape[1], w.shape[2]
+    if not (x.dim() == 3 and out.dim() == 3 and w.dim() == 3 and w.is_contiguous() and w.shape[0] == H
+            and w.dtype == x.dtype and x.stride(2) == 1 and out.stride(2) == 1 and tuple(out.shape[:2]) == (T, H)
+            and x.shape[2] == inner and out.shape[2] == cols and inner <= HEAD_PRODUCT_INNER
+            and (out.dtype == x.dtype or out.dtype == torch.float32)):
+        _fail("head_products: x [T, heads, inner], w [heads, inner, cols], out [T, heads, cols]")
+    _check(_lib().tl_head_products(_ptr(x), c_int64(x.stride(0)), c_int(x.stride(1)), _ptr(w), _ptr(out),
+                                   c_int64(out.stride(0)), c_int(out.stride(1)), c_int(T), c_int(H), c_int(inner),
+                                   c_int(cols), c_int(_dt(x)), c_int(_dt(out)), _stream()), "head_products")
+    return out
+
+
 # ------------------------------------------------------------------ gated delta rule
 DELTA_MAX_DIM = 256     # key channels of a head (csrc/delta_rule.hip)
 DELTA_MAX_TAPS = 16
@@ -1314,6 +1336,44 @@ def delta_recurrence(qn: torch.Tensor, kn: torch.Tensor, vc: torch.Tensor, beta:
                                       c_int64(state.stride(0)), _ptr(cu_seqlens), _ptr(state_slots), _ptr(out),
                                       c_int(R), c_int(heads), c_int(dim), c_int(vdim), _stream()), "delta_recurrence")
     return out
+
+
+DELTA_DECODE_MAX_VDIM = 1024     # a thread per value column in the one-kernel decode step
+
+
+def delta_decode(p: torch.Tensor, conv_off: int, b_off: int, low: torch.Tensor, conv_w: torch.Tensor,
+                 a_log: torch.Tensor, dt_bias: torch.Tensor, w_norm: torch.Tensor, state: torch.Tensor,
+                 saved_off: int, cu_seqlens: torch.Tensor, state_slots: torch.Tensor, z: torch.Tensor, heads: int,
+                 kv_heads: int, dim: int, vdim: int, taps: int, q_scale: float, eps: float) -> torch.Tensor:
+    """A decode step of the delta rule in one kernel (every request brings one token; row t of the
+    operands is request t): what `delta_prepare`, `delta_recurrence` and `head_norm_gate` do, with
+    `low` [T, heads * dim + heads * vdim] float32 = [decay | gate] pre-activations.  The saved
+    convolution inputs are read only: `conv_state_update` follows."""
+    _dev(p, low, conv_w, a_log, dt_bias, w_norm, state, cu_seqlens, state_slots, z)
+    check_delta_sizes(heads, kv_heads, dim, vdim, taps)
+    _rows_2d(p, "projections")
+    _rows_2d(low, "decay and gate pre-activations")
+    _i32(cu_seqlens, state_slots)
+    R = state_slots.numel()
+    channels = 2 * kv_heads * dim + heads * vdim
+    _f32_vec(conv_w, channels * taps, "convolution taps")
+    _f32_vec(a_log, heads, "A_log")
+    _f32_vec(dt_bias, heads * dim, "dt_bias")
+    _f32_vec(w_norm, vdim, "the head norm's weight")
+    if not (p.shape[0] == R and low.shape[0] == R and low.dtype == torch.float32
+            and low.shape[1] >= heads * (dim + vdim) and conv_off + channels <= p.shape[1] and b_off + heads <= p.shape[1]
+            and cu_seqlens.numel() == R + 1 and vdim <= DELTA_DECODE_MAX_VDIM
+            and state.dtype == torch.float32 and state.dim() == 2 and state.is_contiguous()
+            and saved_off + channels * (taps - 1) <= state.shape[1] and heads * dim * vdim <= saved_off
+            and z.dtype == p.dtype and z.is_contiguous() and tuple(z.shape) == (R, heads * vdim)):
+        _fail("delta_decode: shapes do not fit (one row per request)")
+    _check(_lib().tl_delta_decode(_ptr(p), c_int64(p.stride(0)), c_int(conv_off), c_int(b_off), _ptr(low),
+                                  c_int64(low.stride(0)), _ptr(conv_w), _ptr(a_log), _ptr(dt_bias), _ptr(w_norm),
+                                  _ptr(state), c_int64(state.stride(0)), c_int64(saved_off), _ptr(cu_seqlens),
+                                  _ptr(state_slots), _ptr(z), c_int(R), c_int(heads), c_int(kv_heads), c_int(dim),
+                                  c_int(vdim), c_int(taps), c_float(q_scale), c_float(eps), c_int(_dt(p)), _stream()),
+           "delta_decode")
+    return z
 
 
 def head_norm_gate(o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, out: torch.Tensor, heads: int,

@@ -108,6 +108,15 @@ class ChannelDelta(Mixer):
         ops.linear(h, self.w_in, p)
         low = ops.scratch("delta_low", (T, H * D + H * V), torch.float32, dev)
         ops.linear(p[:, self.low_off:self.low_off + self.ra + self.rg], self.w_low, low)
+        z = ops.scratch("delta_gated", (T, H * V), self.dtype, dev)
+        if ctx.max_q_len == 1 and T == ctx.num_requests and V <= ops.DELTA_DECODE_MAX_VDIM:
+            # decoding: every request brings one token; convolutions, recurrence, norm and gate in one kernel
+            ops.delta_decode(p, 0, self.b_off, low, self.conv_w, self.a_log, self.dt_bias, self.w_norm, state,
+                             self.state_size, ctx.cu_seqlens_q, ctx.state_slots, z, H, KH, D, V, self.taps, D ** -0.5,
+                             self.eps)
+            ops.conv_state_update(p, 0, self.channels, state, self.state_size, ctx.cu_seqlens_q, ctx.state_slots,
+                                  self.taps)
+            return self._project_out(z, residual)
         qn = ops.scratch("delta_q", (T * H * D,), torch.float32, dev)
         kn = ops.scratch("delta_k", (T * H * D,), torch.float32, dev)
         dec = ops.scratch("delta_decay", (T * H * D,), torch.float32, dev)
@@ -119,10 +128,13 @@ class ChannelDelta(Mixer):
         ops.conv_state_update(p, 0, self.channels, state, self.state_size, ctx.cu_seqlens_q, ctx.state_slots, self.taps)
         o = ops.scratch("delta_o", (T * H * V,), torch.float32, dev)
         ops.delta_recurrence(qn, kn, vc, beta, dec, state, ctx.cu_seqlens_q, ctx.state_slots, o, H, D, V)
-        z = ops.scratch("delta_gated", (T, H * V), self.dtype, dev)
         ops.head_norm_gate(o, self.w_norm, low[:, H * D:], z, H, V, self.eps)
+        return self._project_out(z, residual)
+
+    def _project_out(self, z, residual):
         if residual is None:
-            return ops.linear(z, self.w_o, ops.scratch("sublayer_out", (T, self.hidden_size), torch.float32, dev))
+            out = ops.scratch("sublayer_out", (z.shape[0], self.hidden_size), torch.float32, z.device)
+            return ops.linear(z, self.w_o, out)
         return ops.linear(z, self.w_o, residual, residual)
 
 

@@ -69,7 +69,7 @@ class LatentAttention(Mixer):
         self.kv_off = _pad8(self.q_rank)
         self.g_off = self.kv_off + (0 if self.shares_cache else _pad8(self.kv_rank + self.rot_dim))
         self.down_width = self.g_off + (_pad8(self.num_heads) if self.gated else 0)
-        self.w_down = self.w_uq = self.w_uk_t = self.w_uv = self.w_o = None
+        self.w_down = self.w_uq = self.w_uk_t = self.w_uv = self.w_o = self.w_uk_few = self.w_uv_few = None
         self.w_dq_norm = self.w_dkv_norm = None
 
     # ---------------------------------------------------------------- declarations
@@ -100,8 +100,12 @@ class LatentAttention(Mixer):
         self.w_dq_norm = tensors[n["dq_norm"]].to(torch.float32).contiguous()
         self.w_uq = tensors[n["uq"]].contiguous()
         # per head the transpose of W_uk: q' = W_uk^T q is a product with [kv_rank, head_dim] weights
-        self.w_uk_t = tensors[n["uk"]].view(H, self.head_dim, self.kv_rank).transpose(1, 2).contiguous()
+        uk = tensors[n["uk"]].view(H, self.head_dim, self.kv_rank)
+        self.w_uk_t = uk.transpose(1, 2).contiguous()
         self.w_uv = tensors[n["uv"]].contiguous()
+        # the same two as [heads, inner, cols], for the one-launch products of steps with few rows
+        self.w_uk_few = uk.contiguous()
+        self.w_uv_few = self.w_uv.view(H, self.value_dim, self.kv_rank).transpose(1, 2).contiguous()
         self.w_o = tensors[n["o"]].contiguous()
 
     def cache_spec(self) -> CacheSpec:
@@ -134,8 +138,12 @@ class LatentAttention(Mixer):
         # [W_uk^T q_unrotated | rotate(q_rotated)] per head, float32
         qa = ops.scratch("latent_qa", (T, H, KR + R), torch.float32, dev)
         q3, qa2 = q.view(T, H, D + R), qa.view(T, H * (KR + R))
-        for n in range(H):
-            ops.linear(q3[:, n, :D], self.w_uk_t[n], qa2[:, n * (KR + R):n * (KR + R) + KR])
+        few = T <= ops.HEAD_PRODUCT_ROWS and max(D, KR) <= ops.HEAD_PRODUCT_INNER
+        if few:
+            ops.head_products(q3[:, :, :D], self.w_uk_few, qa[:, :, :KR])
+        else:
+            for n in range(H):
+                ops.linear(q3[:, n, :D], self.w_uk_t[n], qa2[:, n * (KR + R):n * (KR + R) + KR])
         if R:
             ops.rotate_into(q, H, D + R, D, R, self.rdims, ctx.positions, cos, sin, qa, KR)
         mix = ops.scratch("latent_mix", (T, H, KR), self.dtype, dev)
@@ -143,8 +151,11 @@ class LatentAttention(Mixer):
         ops.latent_attention(qa, latent, rope, ctx.block_tables[cache.group], ctx.req_of_token, ctx.positions, mix,
                              self.scale, gate)
         o = ops.scratch("latent_heads", (T, H * V), self.dtype, dev)
-        for n in range(H):
-            ops.linear(mix[:, n, :], self.w_uv[n * V:(n + 1) * V], o[:, n * V:(n + 1) * V])
+        if few:
+            ops.head_products(mix, self.w_uv_few, o.view(T, H, V))
+        else:
+            for n in range(H):
+                ops.linear(mix[:, n, :], self.w_uv[n * V:(n + 1) * V], o[:, n * V:(n + 1) * V])
         if residual is None:
             return ops.linear(o, self.w_o, ops.scratch("sublayer_out", (T, self.hidden_size), torch.float32, dev))
         return ops.linear(o, self.w_o, residual, residual)
