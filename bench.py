@@ -734,8 +734,13 @@ def kernels_by_name(run):
     evs = [e for e in prof.events() if e.device_type == DeviceType.CUDA and "emcpy" not in e.name and "emset" not in e.name]
     steps = max(1, sum(1 for e in evs if "embedding_kernel" in e.name))
     out = {}
+    import re
     for e in evs:
-        name = e.name.split("<")[0].split("(")[0].replace("(anonymous namespace)::", "").replace("void ", "").strip()
+        m = re.match(r"_ZN12_GLOBAL__N_1(\d+)", e.name)          # a kernel of the library's unnamed namespace
+        if m:
+            name = e.name[m.end():m.end() + int(m.group(1))]
+        else:
+            name = e.name.split("<")[0].split("(")[0].replace("void ", "").strip() or "(unnamed)"
         t, n = out.get(name, (0.0, 0))
         out[name] = (t + (e.time_range.end - e.time_range.start), n + 1)
     return {k: {"us": round(t / steps, 1), "launches": round(n / steps, 1)} for k, (t, n) in sorted(out.items(), key=lambda kv: -kv[1][0])}

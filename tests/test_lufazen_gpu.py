@@ -219,15 +219,18 @@ def _paged(rows: torch.Tensor, table, block, n_blocks, dtype):
     return pages
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, "matrix cores", "matrix cores, split keys"])
 def test_latent_attention_finds_one_key(dtype):
     """One query per place of interest is aligned with the latent of one key (and scaled so that this
     score stands out): the result must be that key's latent.  Keys at the first positions, at both
     sides of page edges, hundreds of tokens back, the query's own position; and the position behind
     the query, which the mask must hide however large its score is."""
     from tiny_llm_amd.kernels import ops
+    flash = isinstance(dtype, str)
+    splits = 3 if flash and "split" in dtype else 1
+    dtype = torch.bfloat16 if flash else dtype
     g = torch.Generator().manual_seed(5)
-    n, kv_rank, rot, block, heads = 700, 40, 8, 16, 3
+    n, kv_rank, rot, block, heads = 700, 48 if flash else 40, 8, 16, 3
     lat = torch.randn(n, kv_rank, generator=g)
     lat = lat / lat.norm(dim=1, keepdim=True)
     rope = torch.randn(n, rot, generator=g) * 0.1
@@ -245,8 +248,14 @@ def test_latent_attention_finds_one_key(dtype):
     positions = torch.tensor([c[0] for c in cases], dtype=torch.int32, device="cuda")
     bt = torch.tensor([table + [0] * (64 - len(table))], dtype=torch.int32, device="cuda")
     out = torch.empty(T, heads, kv_rank, dtype=dtype, device="cuda")
-    ops.latent_attention(qa.cuda(), pages_l, pages_r, bt, torch.zeros(T, dtype=torch.int32, device="cuda"), positions,
-                         out, 1.0)
+    if flash:
+        # every query a request of its own (the same pages under every row of the table), as in a decode step
+        part = torch.empty(splits * T * heads * (kv_rank + 2), device="cuda") if splits > 1 else None
+        ops.latent_flash(qa.cuda(), pages_l, pages_r, bt.repeat(T, 1).contiguous(), None, positions, out, 1.0, None,
+                         splits, part)
+    else:
+        ops.latent_attention(qa.cuda(), pages_l, pages_r, bt, torch.zeros(T, dtype=torch.int32, device="cuda"),
+                             positions, out, 1.0)
     # the plain softmax over the visible keys
     lat_r, rope_r = lat.to(dtype).double(), rope.to(dtype).double()
     for i, (pos, key) in enumerate(cases):
@@ -255,6 +264,8 @@ def test_latent_attention_finds_one_key(dtype):
         got = out[i, 0].double().cpu()
         assert torch.isfinite(got).all()
         assert (got - want).abs().max() < (2e-5 if dtype == torch.float32 else 1e-2), (pos, key)
+        for h in range(1, heads):
+            assert torch.equal(out[i, h], out[i, 0])
 
 
 def test_delta_rule_state_over_slots_and_tiny_portions():

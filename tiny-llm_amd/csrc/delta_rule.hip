@@ -110,48 +110,94 @@ __global__ void conv_state_update_kernel(const T* __restrict__ p, int64_t p_stri
     if (i < taps - 1) saved[i] = next[i];
 }
 
-// The recurrence.  One wave per (request, head, 64 value columns); lane j keeps column j of S in
-// registers and walks the request's tokens of this step in order.  q, k and the decay of a token
-// are the same for all lanes.
-template <int DIM>
+// The recurrence.  One wave per (request, head, 16 value columns): lane (s, c) keeps rows
+// [s * DS, (s + 1) * DS) of column c of S in registers (four slices of the key channels side by side,
+// 16 lanes each), so a token costs DS steps and two sums over the four slices instead of `dim` steps.
+// The wave walks the request's tokens of this step in order, kCh at a time: q, k, decay, v and beta of a
+// chunk go through LDS, and the next chunk's are requested before this one is worked on.
+constexpr int kCh = 16;           // tokens per staged chunk
+constexpr int kCols = 16;         // value columns per wave
+template <int DS>
 __global__ __launch_bounds__(TL_WAVE) void delta_recurrence_kernel(
     const float* __restrict__ qn, const float* __restrict__ kn, const float* __restrict__ vc,
     const float* __restrict__ beta, const float* __restrict__ decay, float* __restrict__ state, int64_t state_stride,
     const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ state_slots, float* __restrict__ out,
     int heads, int dim, int vdim) {
-  const int r = blockIdx.x, h = blockIdx.y;
-  const int col = blockIdx.z * TL_WAVE + threadIdx.x;
+  constexpr int DP = 4 * DS;                      // key channels, padded
+  constexpr int PER = kCh * DP / TL_WAVE;         // floats of one staged array a lane moves per chunk
+  __shared__ float ks[kCh][DP], qs[kCh][DP], gs[kCh][DP], vs[kCh][kCols], bs[kCh];
+  const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int s = lane / kCols, c = lane % kCols;
+  const int col = blockIdx.z * kCols + c;
   const int t0 = cu_seqlens[r], t1 = cu_seqlens[r + 1];
-  if (t1 <= t0 || col >= vdim) return;        // a padding request owns no state
+  if (t1 <= t0) return;                           // a padding request owns no state
+  const bool live = col < vdim;
   float* S_mem = state + (int64_t)state_slots[r] * state_stride + (int64_t)h * dim * vdim + col;
-  float S[DIM];
+  float S[DS];
 #pragma unroll
-  for (int i = 0; i < DIM; ++i) S[i] = i < dim ? S_mem[(int64_t)i * vdim] : 0.f;
-  for (int t = t0; t < t1; ++t) {
-    const int64_t base = (int64_t)t * heads + h;
-    const float* __restrict__ k = kn + base * dim;
-    const float* __restrict__ q = qn + base * dim;
-    const float* __restrict__ g = decay + base * dim;
-    float sk = 0.f;
+  for (int i = 0; i < DS; ++i) S[i] = (live && s * DS + i < dim) ? S_mem[(int64_t)(s * DS + i) * vdim] : 0.f;
+
+  float rk[PER], rq[PER], rg[PER], rv[(kCh * kCols) / TL_WAVE], rb = 0.f;
+  // element e of a staged array: token e / DP of the chunk, channel e % DP (channels beyond dim: k = q = 0, g = 1)
+  auto fetch = [&](int tc) {
 #pragma unroll
-    for (int i = 0; i < DIM; ++i)
-      if (i < dim) {
+    for (int j = 0; j < PER; ++j) {
+      const int e = j * TL_WAVE + lane, tt = e / DP, i = e % DP;
+      const bool ok = tc + tt < t1 && i < dim;
+      const int64_t at = ((int64_t)(tc + tt) * heads + h) * dim + i;
+      rk[j] = ok ? kn[at] : 0.f;
+      rq[j] = ok ? qn[at] : 0.f;
+      rg[j] = ok ? decay[at] : 1.f;
+    }
+#pragma unroll
+    for (int j = 0; j < (kCh * kCols) / TL_WAVE; ++j) {
+      const int e = j * TL_WAVE + lane, tt = e / kCols, cc = e % kCols;
+      const int vcol = blockIdx.z * kCols + cc;
+      rv[j] = (tc + tt < t1 && vcol < vdim) ? vc[((int64_t)(tc + tt) * heads + h) * vdim + vcol] : 0.f;
+    }
+    rb = (lane < kCh && tc + lane < t1) ? beta[(int64_t)(tc + lane) * heads + h] : 0.f;
+  };
+  fetch(t0);
+  for (int tc = t0; tc < t1; tc += kCh) {
+    __syncthreads();                              // the chunk before has been read
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int e = j * TL_WAVE + lane;
+      (&ks[0][0])[e] = rk[j];
+      (&qs[0][0])[e] = rq[j];
+      (&gs[0][0])[e] = rg[j];
+    }
+#pragma unroll
+    for (int j = 0; j < (kCh * kCols) / TL_WAVE; ++j) (&vs[0][0])[j * TL_WAVE + lane] = rv[j];
+    if (lane < kCh) bs[lane] = rb;
+    __syncthreads();
+    if (tc + kCh < t1) fetch(tc + kCh);           // on its way while this chunk is worked on
+    const int n = min(kCh, t1 - tc);
+    for (int tt = 0; tt < n; ++tt) {
+      const float* k = &ks[tt][s * DS];
+      const float* q = &qs[tt][s * DS];
+      const float* g = &gs[tt][s * DS];
+      float sk = 0.f;
+#pragma unroll
+      for (int i = 0; i < DS; ++i) {
         S[i] *= g[i];
         sk = fmaf(S[i], k[i], sk);
       }
-    const float u = beta[base] * (vc[base * vdim + col] - sk);
-    float o = 0.f;
+      sk = sum_over_rows(sk);
+      const float u = bs[tt] * (vs[tt][c] - sk);
+      float o = 0.f;
 #pragma unroll
-    for (int i = 0; i < DIM; ++i)
-      if (i < dim) {
+      for (int i = 0; i < DS; ++i) {
         S[i] = fmaf(k[i], u, S[i]);
         o = fmaf(S[i], q[i], o);
       }
-    out[base * vdim + col] = o;
+      o = sum_over_rows(o);
+      if (s == 0 && live) out[((int64_t)(tc + tt) * heads + h) * vdim + col] = o;
+    }
   }
 #pragma unroll
-  for (int i = 0; i < DIM; ++i)
-    if (i < dim) S_mem[(int64_t)i * vdim] = S[i];
+  for (int i = 0; i < DS; ++i)
+    if (live && s * DS + i < dim) S_mem[(int64_t)(s * DS + i) * vdim] = S[i];
 }
 
 // z[t, h, :] = w * o[t, h, :] / sqrt(mean(o[t, h, :]^2) + eps) * sigmoid(gate[t, h, :]); one wave per (t, h).
@@ -296,17 +342,17 @@ int tl_delta_recurrence(const float* qn, const float* kn, const float* vc, const
                         float* state, int64_t state_stride, const int32_t* cu_seqlens, const int32_t* state_slots,
                         float* out, int n_requests, int heads, int dim, int vdim, hipStream_t stream) {
   if (n_requests <= 0) return TL_OK;
-  if (heads <= 0 || heads > 65535 || dim <= 0 || dim > kMaxDim || vdim <= 0 || (vdim + 63) / 64 > 65535)
+  if (heads <= 0 || heads > 65535 || dim <= 0 || dim > kMaxDim || vdim <= 0 || (vdim + kCols - 1) / kCols > 65535)
     return TL_ERR_ARG;
-  dim3 g(n_requests, heads, (vdim + TL_WAVE - 1) / TL_WAVE), b(TL_WAVE);
-#define TL_REC(D)                                                                                                    \
-  hipLaunchKernelGGL(delta_recurrence_kernel<D>, g, b, 0, stream, qn, kn, vc, beta, decay, state, state_stride,      \
+  dim3 g(n_requests, heads, (vdim + kCols - 1) / kCols), b(TL_WAVE);
+#define TL_REC(DS)                                                                                                   \
+  hipLaunchKernelGGL(delta_recurrence_kernel<DS>, g, b, 0, stream, qn, kn, vc, beta, decay, state, state_stride,     \
                      cu_seqlens, state_slots, out, heads, dim, vdim)
-  if (dim <= 16) TL_REC(16);
-  else if (dim <= 32) TL_REC(32);
-  else if (dim <= 64) TL_REC(64);
-  else if (dim <= 128) TL_REC(128);
-  else TL_REC(256);
+  if (dim <= 16) TL_REC(4);
+  else if (dim <= 32) TL_REC(8);
+  else if (dim <= 64) TL_REC(16);
+  else if (dim <= 128) TL_REC(32);
+  else TL_REC(64);
 #undef TL_REC
   return tl_launch_status();
 }

@@ -152,6 +152,230 @@ __global__ __launch_bounds__(TL_WAVE) void latent_attention_kernel(
   }
 }
 
+// ===================================================================== bfloat16 on MFMA
+// latent_flash_bf16_kernel: the same function on the matrix cores.  A workgroup of four waves owns a
+// tile of 16 query rows of ONE request: `tpt` consecutive tokens times up to 16 heads (row = token *
+// hg + head, hg = min(heads, 16)); every head scores against the same cached rows [c | kr], so 16 heads
+// of one token fill a matrix tile.  The waves deal the request's 16-key tiles out between them (and
+// `n_splits` workgroups split them further: decoding with few requests), each with its own running
+// (max, sum, output), merged at the end.  Scores are computed transposed, S^T = [C | Kr] Q^T with
+// v_mfma_f32_16x16x32_bf16 (keys straight from memory into operands), so that a lane holds four scores
+// of ONE query row and the softmax needs two exchanges; the probabilities are then already the operand
+// of O^T = C^T P^T (v_mfma_f32_16x16x16_bf16), whose other operand comes from the wave's own LDS copy
+// of the key tile's latents through the transposing read.  The queries [W_uk^T q | q_rot] enter the score
+// product as a sum of two bfloat16 terms (staged once per tile), so nothing of their float32 value is
+// lost against float32 scores over bfloat16 keys; scores, softmax and sums are float32.
+constexpr int LF_WAVES = 4;
+constexpr int LF_MAXKS = 18;        // (512 + 64) / 32 steps of the score product
+constexpr int LF_MAXDT = 32;        // 512 / 16 tiles of the output
+constexpr int LF_PAD = 8;           // elements added to an LDS row (rows 16 bytes apart in the banks)
+constexpr float kNegBig = -1.0e30f; // "no key yet": finite, so exp2(m - m') never sees inf - inf
+typedef short lf_i16x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ bf16x4 lf_read_transposed(const bf16_t* p) {
+  return __builtin_bit_cast(bf16x4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) lf_i16x4*)p));
+}
+__device__ __forceinline__ void lf_wave_sync() {      // a wave's LDS operations are carried out in order
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+__global__ __launch_bounds__(LF_WAVES * TL_WAVE) void latent_flash_bf16_kernel(
+    const float* __restrict__ qa, const bf16_t* __restrict__ latent, const bf16_t* __restrict__ rope,
+    const int32_t* __restrict__ block_tables, int max_blocks, const int32_t* __restrict__ tile_req,
+    const int32_t* __restrict__ tile_tok0, const int32_t* __restrict__ tile_ntok,
+    const int32_t* __restrict__ positions, const bf16_t* __restrict__ gate, int64_t gate_stride,
+    bf16_t* __restrict__ out, float* __restrict__ part, int n_tokens, int heads, int tpt, int kv_rank, int rot,
+    int block_size, float scale, int n_splits) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lf_smem[];
+  const int wave = threadIdx.x / TL_WAVE, lane = threadIdx.x % TL_WAVE, g = lane / 16, c = lane % 16;
+  const int tile = blockIdx.x, head0 = blockIdx.y * 16, split = blockIdx.z;
+  const int hg = min(heads, 16);
+  const int r = tile_req ? tile_req[tile] : tile;
+  const int tok0 = tile_tok0 ? tile_tok0[tile] : tile;
+  const int ntok = tile_ntok ? tile_ntok[tile] : 1;
+  if (ntok <= 0) return;                              // a padding tile
+  const int W = kv_rank + rot, WP = (W + 31) / 32 * 32, KS = WP / 32, KDT = kv_rank / 16;
+  const int QS = WP + LF_PAD, VS = kv_rank + LF_PAD;
+  bf16_t* Ql = (bf16_t*)lf_smem;                     // the queries' upper terms, then their lower terms
+  bf16_t* Qlo = Ql + 16 * QS;
+  bf16_t* Vl = Qlo + 16 * QS + wave * 16 * VS;
+  const int32_t* bt = block_tables + (int64_t)r * max_blocks;
+
+  // the query tile as q = hi + lo in bfloat16; rows without a query and dims beyond W are zero
+  for (int e = threadIdx.x; e < 16 * WP; e += LF_WAVES * TL_WAVE) {
+    const int row = e / WP, d = e - row * WP;
+    const int tt = row / hg, h = head0 + row % hg;
+    float v = 0.f;
+    if (tt < ntok && tt < tpt && h < heads && d < W) v = qa[((int64_t)(tok0 + tt) * heads + h) * W + d];
+    const bf16_t hi = (bf16_t)v;
+    Ql[row * QS + d] = hi;
+    Qlo[row * QS + d] = (bf16_t)(v - (float)hi);
+  }
+  const int my_tt = c / hg, my_h = head0 + c % hg;
+  const bool row_valid = my_tt < ntok && my_tt < tpt && my_h < heads;
+  const int my_tok = tok0 + min(my_tt, ntok - 1);
+  const int pos = positions[my_tok];
+  const int kv_end = positions[tok0 + ntok - 1] + 1;  // what the tile's last token sees
+  const int n_kt = (kv_end + 15) / 16;
+  const float c_log2 = scale * 1.44269504088896f;
+  __syncthreads();
+
+  bf16x8 kop[LF_MAXKS];
+  auto fetch = [&](int kt) {
+    const int j = min(kt * 16 + c, kv_end - 1);       // keys beyond the end read a row that exists
+    const int64_t slot = (int64_t)bt[j / block_size] * block_size + (j % block_size);
+#pragma unroll
+    for (int ks = 0; ks < LF_MAXKS; ++ks) {
+      if (ks < KS) {
+        const int d0 = ks * 32 + g * 8;
+        if (d0 < kv_rank) kop[ks] = *(const bf16x8*)(latent + slot * kv_rank + d0);
+        else if (d0 - kv_rank < rot) kop[ks] = *(const bf16x8*)(rope + slot * rot + (d0 - kv_rank));
+        else kop[ks] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+      }
+    }
+  };
+  float m_run = kNegBig, l_run = 0.f;
+  f32x4 o[LF_MAXDT];
+#pragma unroll
+  for (int dt = 0; dt < LF_MAXDT; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  const int first = split * LF_WAVES + wave, stride = n_splits * LF_WAVES;
+  if (first < n_kt) fetch(first);
+  for (int kt = first; kt < n_kt; kt += stride) {
+    // the tile's latents into this wave's LDS area (row c, the chunk this lane holds), and the scores
+    f32x4 sc = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < LF_MAXKS; ++ks) {
+      if (ks < KS) {
+        const int d0 = ks * 32 + g * 8;
+        if (d0 < kv_rank) *(bf16x8*)(Vl + c * VS + d0) = kop[ks];
+        const bf16x8 qf = *(const bf16x8*)(Ql + c * QS + d0), ql = *(const bf16x8*)(Qlo + c * QS + d0);
+        sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop[ks], qf, sc, 0, 0, 0);
+        sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop[ks], ql, sc, 0, 0, 0);
+      }
+    }
+    if (kt + stride < n_kt) fetch(kt + stride);       // on its way while this tile is worked on
+    lf_wave_sync();
+    // sc[i] = S^T[key kt*16 + g*4 + i][row c]
+    float m_tile = kNegBig;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int j = kt * 16 + g * 4 + i;
+      const bool ok = row_valid && j <= pos;
+      sc[i] = ok ? sc[i] * c_log2 : -INFINITY;
+      m_tile = fmaxf(m_tile, sc[i]);
+    }
+    m_tile = max_over_rows(m_tile);
+    const float m_new = fmaxf(m_run, m_tile);
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+    float psum = 0.f;
+    bf16x4 pb;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float p = __builtin_amdgcn_exp2f(sc[i] - m_new);
+      psum += p;
+      pb[i] = (bf16_t)p;
+    }
+    psum = sum_over_rows(psum);
+    l_run = l_run * alpha + psum;
+    m_run = m_new;
+    // lane s of a group names keys g*4 + s/4, dims dt*16 + 4*(s%4) ..; it receives keys g*4 .. g*4+3 of dim dt*16 + s
+    const bf16_t* vsrc = Vl + (g * 4 + c / 4) * VS + 4 * (c % 4);
+#pragma unroll
+    for (int dt = 0; dt < LF_MAXDT; ++dt) {
+      if (dt < KDT) {
+        const bf16x4 vf = lf_read_transposed(vsrc + dt * 16);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[dt][i] *= alpha;
+        o[dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(lf_i16x4, vf),
+                                                          __builtin_bit_cast(lf_i16x4, pb), o[dt], 0, 0, 0);
+      }
+    }
+    lf_wave_sync();                                   // the reads are done before the next tile is written
+  }
+  __syncthreads();                                    // the merge writes over the staging areas
+
+  // merge: waves 1 to 3 leave (O, m, l) in turn, wave 0 adds them to its own; o[dt][i] = O[row c][dt*16 + g*4 + i]
+  float* Mg = (float*)(Qlo + 16 * QS);
+  const int MROW = kv_rank + 2;
+  for (int src = 1; src < LF_WAVES; ++src) {
+    if (wave == src) {
+#pragma unroll
+      for (int dt = 0; dt < LF_MAXDT; ++dt)
+        if (dt < KDT) *(f32x4*)(Mg + c * MROW + dt * 16 + g * 4) = o[dt];
+      if (g == 0) {
+        Mg[c * MROW + kv_rank] = m_run;
+        Mg[c * MROW + kv_rank + 1] = l_run;
+      }
+    }
+    __syncthreads();
+    if (wave == 0) {
+      const float m_o = Mg[c * MROW + kv_rank], l_o = Mg[c * MROW + kv_rank + 1];
+      const float m_new = fmaxf(m_run, m_o);
+      const float a = __builtin_amdgcn_exp2f(m_run - m_new), b = __builtin_amdgcn_exp2f(m_o - m_new);
+#pragma unroll
+      for (int dt = 0; dt < LF_MAXDT; ++dt)
+        if (dt < KDT) {
+          const f32x4 other = *(const f32x4*)(Mg + c * MROW + dt * 16 + g * 4);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) o[dt][i] = o[dt][i] * a + other[i] * b;
+        }
+      l_run = l_run * a + l_o * b;
+      m_run = m_new;
+    }
+    __syncthreads();
+  }
+  if (wave != 0 || !row_valid) return;
+  if (n_splits > 1) {                                 // unnormalised, for latent_combine_kernel
+    float* prow = part + (((int64_t)split * n_tokens + my_tok) * heads + my_h) * MROW;
+#pragma unroll
+    for (int dt = 0; dt < LF_MAXDT; ++dt)
+      if (dt < KDT) *(f32x4*)(prow + dt * 16 + g * 4) = o[dt];
+    if (g == 0) {
+      prow[kv_rank] = m_run;
+      prow[kv_rank + 1] = l_run;
+    }
+    return;
+  }
+  float f = l_run > 0.f ? 1.f / l_run : 0.f;
+  if (gate) f /= 1.f + expf(-(float)gate[(int64_t)my_tok * gate_stride + my_h]);
+  bf16_t* orow = out + ((int64_t)my_tok * heads + my_h) * kv_rank + g * 4;
+#pragma unroll
+  for (int dt = 0; dt < LF_MAXDT; ++dt)
+    if (dt < KDT) {
+      bf16x4 v4;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v4[i] = (bf16_t)(o[dt][i] * f);
+      *(bf16x4*)(orow + dt * 16) = v4;
+    }
+}
+
+// Merges the partial results of `n_splits` workgroups: one wave per (token, head); maxima are in
+// units of log2 e; a split without keys has l = 0.
+__global__ __launch_bounds__(TL_WAVE) void latent_combine_kernel(const float* __restrict__ part,
+                                                                 const bf16_t* __restrict__ gate, int64_t gate_stride,
+                                                                 bf16_t* __restrict__ out, int n_tokens, int heads,
+                                                                 int kv_rank, int n_splits) {
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int MROW = kv_rank + 2;
+  const int64_t row = (int64_t)t * heads + h, step = (int64_t)n_tokens * heads;
+  float M = kNegBig;
+  for (int s = 0; s < n_splits; ++s) M = fmaxf(M, part[(row + s * step) * MROW + kv_rank]);
+  float L = 0.f;
+  for (int s = 0; s < n_splits; ++s)
+    L += __builtin_amdgcn_exp2f(part[(row + s * step) * MROW + kv_rank] - M) * part[(row + s * step) * MROW + kv_rank + 1];
+  float f = L > 0.f ? 1.f / L : 0.f;
+  if (gate) f /= 1.f + expf(-(float)gate[(int64_t)t * gate_stride + h]);
+  for (int d = lane; d < kv_rank; d += TL_WAVE) {
+    float acc = 0.f;
+    for (int s = 0; s < n_splits; ++s)
+      acc += __builtin_amdgcn_exp2f(part[(row + s * step) * MROW + kv_rank] - M) * part[(row + s * step) * MROW + d];
+    out[row * kv_rank + d] = (bf16_t)(acc * f);
+  }
+}
+
 // Small products per head for steps of few rows: out[t, h, n] = sum_k w[h, k, n] * in[t, h, k].
 // The weights lie [heads, inner, cols], so that the threads of a workgroup (one per output column)
 // read them in whole lines; a workgroup takes up to kRows rows at a time, whose inputs it keeps in LDS.
@@ -235,6 +459,38 @@ int tl_latent_attention(const float* qa, const void* latent, const void* rope, c
                                           (const T*)rope, block_tables, max_blocks, req_of_token, positions,
                                           (const T*)gate, gate_stride, (T*)out, heads, kv_rank, rot, block_size,
                                           scale);)
+  return tl_launch_status();
+}
+
+// bfloat16 on the matrix cores.  Tiles: `tpt` = 16 / min(heads, 16) tokens of one request each (null
+// arrays: tile i is token i of request i).  n_splits > 1: `part` is scratch of
+// n_splits * n_tokens * heads * (kv_rank + 2) floats.  kv_rank a multiple of 16 up to 512, rot a multiple of 8 up to 64.
+int tl_latent_flash(const float* qa, const void* latent, const void* rope, const int32_t* block_tables, int max_blocks,
+                    const int32_t* tile_req, const int32_t* tile_tok0, const int32_t* tile_ntok,
+                    const int32_t* positions, const void* gate, int64_t gate_stride, void* out, float* part,
+                    int n_tiles, int n_tokens, int heads, int tpt, int kv_rank, int rot, int block_size, float scale,
+                    int n_splits, hipStream_t stream) {
+  if (n_tiles <= 0 || n_tokens <= 0) return TL_OK;
+  if (heads <= 0 || kv_rank <= 0 || kv_rank % 16 || kv_rank > 16 * LF_MAXDT || rot < 0 || rot % 8 ||
+      kv_rank + rot > 32 * LF_MAXKS || block_size <= 0 || max_blocks <= 0 || n_splits < 1 || n_splits > 65535 ||
+      tpt != 16 / (heads < 16 ? heads : 16) || (n_splits > 1 && !part) || (heads + 15) / 16 > 65535)
+    return TL_ERR_ARG;
+  const int WP = (kv_rank + rot + 31) / 32 * 32;
+  const size_t lds = (size_t)2 * 16 * (WP + LF_PAD) * 2 + (size_t)LF_WAVES * 16 * (kv_rank + LF_PAD) * 2;
+  static int granted = 0;                 // the most dynamic LDS asked for so far (the default limit is 64 KB)
+  if ((int)lds > granted) {
+    if (hipFuncSetAttribute((const void*)latent_flash_bf16_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)lds) != hipSuccess)
+      return TL_ERR_LAUNCH;
+    granted = (int)lds;
+  }
+  dim3 g(n_tiles, (heads + 15) / 16, n_splits), b(LF_WAVES * TL_WAVE);
+  hipLaunchKernelGGL(latent_flash_bf16_kernel, g, b, lds, stream, qa, (const bf16_t*)latent, (const bf16_t*)rope,
+                     block_tables, max_blocks, tile_req, tile_tok0, tile_ntok, positions, (const bf16_t*)gate,
+                     gate_stride, (bf16_t*)out, part, n_tokens, heads, tpt, kv_rank, rot, block_size, scale, n_splits);
+  if (n_splits > 1)
+    hipLaunchKernelGGL(latent_combine_kernel, dim3(n_tokens, heads), dim3(TL_WAVE), 0, stream, part,
+                       (const bf16_t*)gate, gate_stride, (bf16_t*)out, n_tokens, heads, kv_rank, n_splits);
   return tl_launch_status();
 }
 

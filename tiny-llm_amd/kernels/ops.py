@@ -1228,6 +1228,68 @@ def latent_attention(qa: torch.Tensor, latent: torch.Tensor, rope: Optional[torc
     return out
 
 
+def latent_flash_supported(dtype: torch.dtype, kv_rank: int, rot: int) -> bool:
+    """Whether the matrix-core kernel takes these sizes (bfloat16 caches; else the general kernel runs)."""
+    return dtype == torch.bfloat16 and kv_rank % 16 == 0 and 0 < kv_rank <= LATENT_MAX_RANK and rot % 8 == 0 \
+        and 0 <= rot and kv_rank + rot <= 576
+
+
+def latent_key_splits(groups: int, max_seq_len: int) -> int:
+    """Into how many workgroups the keys of one query tile are split: enough to give the chip a round
+    of workgroups when the step has few tiles (decoding), never fewer than 64 keys a workgroup."""
+    if groups <= 0 or groups >= 256:
+        return 1
+    return max(1, min(256 // groups, -(-max_seq_len // 64), 64))
+
+
+def latent_flash(qa: torch.Tensor, latent: torch.Tensor, rope: Optional[torch.Tensor], block_tables: torch.Tensor,
+                 tiles, positions: torch.Tensor, out: torch.Tensor, scale: float, gate: Optional[torch.Tensor] = None,
+                 n_splits: int = 1, scratch_buf: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """`latent_attention` on the matrix cores (bfloat16 caches).  tiles = (tile_req, tile_tok0, tile_ntok)
+    with at most 16 // min(heads, 16) tokens of one request each, or None: tile i is token i of request i.
+    n_splits > 1: scratch_buf holds n_splits * T * heads * (kv_rank + 2) floats."""
+    _dev(qa, latent, rope, block_tables, positions, out, gate, scratch_buf)
+    _i32(block_tables, positions)
+    T, H, W = qa.shape
+    kv_rank = latent.shape[-1]
+    rot = W - kv_rank
+    if not latent_flash_supported(latent.dtype, kv_rank, rot):
+        _fail(f"latent_flash takes bfloat16 latents of a multiple of 16 up to 512 and rotated dims of a multiple of 8; got {kv_rank}, {rot}")
+    if not (qa.dtype == torch.float32 and qa.is_contiguous() and latent.dim() == 3 and latent.is_contiguous()
+            and block_tables.dim() == 2 and positions.numel() == T):
+        _fail("latent_flash: queries are contiguous float32 [T, heads, kv_rank + rot], the cache [blocks, block_size, kv_rank]")
+    if rot and not (rope is not None and rope.dtype == latent.dtype and rope.is_contiguous()
+                    and tuple(rope.shape) == (*latent.shape[:2], rot)):
+        _fail("latent_flash: the rotated-key cache must be [blocks, block_size, rot] of the cache's type")
+    if not (out.dtype == latent.dtype and out.is_contiguous() and tuple(out.shape) == (T, H, kv_rank)):
+        _fail("latent_flash: the output is contiguous [T, heads, kv_rank] of the cache's type")
+    if gate is not None and not (gate.dtype == latent.dtype and gate.dim() == 2 and gate.stride(1) == 1
+                                 and tuple(gate.shape) == (T, H)):
+        _fail("latent_flash: the gate is [T, heads] of the cache's type")
+    if tiles is None:
+        if not (block_tables.shape[0] >= T):
+            _fail("latent_flash: without tile lists every token is a request of its own")
+        treq = ttok = tn = None
+        n_tiles = T
+    else:
+        treq, ttok, tn = tiles
+        _dev(treq, ttok, tn)
+        _i32(treq, ttok, tn)
+        n_tiles = treq.numel()
+        if not (ttok.numel() == n_tiles and tn.numel() == n_tiles):
+            _fail("latent_flash: the three tile lists have one length")
+    if n_splits > 1 and not (scratch_buf is not None and scratch_buf.dtype == torch.float32 and scratch_buf.is_contiguous()
+                             and scratch_buf.numel() >= n_splits * T * H * (kv_rank + 2)):
+        _fail("latent_flash: split keys need float32 scratch of n_splits * T * heads * (kv_rank + 2)")
+    _check(_lib().tl_latent_flash(_ptr(qa), _ptr(latent, 16), _ptr(rope, 16), _ptr(block_tables),
+                                  c_int(block_tables.shape[1]), _ptr(treq), _ptr(ttok), _ptr(tn), _ptr(positions),
+                                  _ptr(gate), c_int64(gate.stride(0) if gate is not None else 0), _ptr(out, 8),
+                                  _ptr(scratch_buf, 16), c_int(n_tiles), c_int(T), c_int(H), c_int(16 // min(H, 16)),
+                                  c_int(kv_rank), c_int(rot), c_int(latent.shape[1]), c_float(scale),
+                                  c_int(n_splits), _stream()), "latent_flash")
+    return out
+
+
 HEAD_PRODUCT_ROWS = 32      # up to this many rows the per-head products of a step run as ONE launch
 HEAD_PRODUCT_INNER = 1024
 

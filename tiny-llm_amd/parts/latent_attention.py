@@ -148,8 +148,21 @@ class LatentAttention(Mixer):
             ops.rotate_into(q, H, D + R, D, R, self.rdims, ctx.positions, cos, sin, qa, KR)
         mix = ops.scratch("latent_mix", (T, H, KR), self.dtype, dev)
         gate = down[:, self.g_off:self.g_off + H] if self.gated else None
-        ops.latent_attention(qa, latent, rope, ctx.block_tables[cache.group], ctx.req_of_token, ctx.positions, mix,
-                             self.scale, gate)
+        if ops.latent_flash_supported(self.dtype, KR, R):
+            # bfloat16: on the matrix cores, 16 heads of a token (or 16 / heads tokens) a tile
+            decode = ctx.max_q_len == 1 and T == ctx.num_requests
+            tpt = 16 // min(H, 16)
+            tiles = None if decode else ctx.attention_tiles(tpt)
+            n_tiles = T if decode else tiles[0].numel()
+            n_splits = ops.latent_key_splits(n_tiles * -(-H // 16), ctx.max_seq_len)
+            part = None
+            if n_splits > 1:
+                part = ops.scratch("attention_partials", (n_splits * T * H * (KR + 2),), torch.float32, dev)
+            ops.latent_flash(qa, latent, rope, ctx.block_tables[cache.group], tiles, ctx.positions, mix, self.scale,
+                             gate, n_splits, part)
+        else:
+            ops.latent_attention(qa, latent, rope, ctx.block_tables[cache.group], ctx.req_of_token, ctx.positions,
+                                 mix, self.scale, gate)
         o = ops.scratch("latent_heads", (T, H * V), self.dtype, dev)
         if few:
             ops.head_products(mix, self.w_uv_few, o.view(T, H, V))
