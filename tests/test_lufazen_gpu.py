@@ -366,3 +366,20 @@ def test_sublayer_kernels():
     lg = (torch.randn(5, 33, generator=g) * 40).cuda()
     want = 25.0 * torch.tanh(lg.cpu().double() / 25.0)
     assert (ops.softcap(lg, 25.0).cpu().double() - want).abs().max() < 1e-4
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_head_products(dtype):
+    """The per-head products of steps with few rows, on views into wider rows, against an einsum."""
+    from tiny_llm_amd.kernels import ops
+    g = torch.Generator().manual_seed(2)
+    for T, H, K, N, extra in ((1, 3, 24, 40, 8), (5, 2, 40, 16, 0), (11, 4, 128, 72, 16), (8, 1, 520, 33, 0)):
+        x = torch.randn(T, H, K + extra, generator=g).to(dtype).cuda()
+        w = (torch.randn(H, K, N, generator=g) / K ** 0.5).to(dtype).cuda()
+        want = torch.einsum("thk,hkn->thn", x[:, :, :K].double().cpu(), w.double().cpu())
+        for out_dtype in {dtype, torch.float32}:
+            out = torch.full((T, H, N + extra), float("nan"), dtype=out_dtype, device="cuda")
+            ops.head_products(x[:, :, :K], w, out[:, :, :N])
+            tol = 1e-5 if out_dtype == torch.float32 else 2e-2
+            assert (out[:, :, :N].double().cpu() - want).abs().max() < tol
+            assert extra == 0 or torch.isnan(out[:, :, N:]).all()      # nothing is written beside the view

@@ -110,20 +110,23 @@ __global__ void conv_state_update_kernel(const T* __restrict__ p, int64_t p_stri
     if (i < taps - 1) saved[i] = next[i];
 }
 
-// The recurrence.  One wave per (request, head, 16 value columns): lane (s, c) keeps rows
-// [s * DS, (s + 1) * DS) of column c of S in registers (four slices of the key channels side by side,
-// 16 lanes each), so a token costs DS steps and two sums over the four slices instead of `dim` steps.
+// The recurrence.  One wave per (request, head, 8 value columns): lane (s, c) keeps rows
+// [s * DS, (s + 1) * DS) of column c of S in registers (eight slices of the key channels side by side,
+// 8 lanes each), so a token costs DS steps and two sums over the eight slices instead of `dim` steps.
 // The wave walks the request's tokens of this step in order, kCh at a time: q, k, decay, v and beta of a
 // chunk go through LDS, and the next chunk's are requested before this one is worked on.
 constexpr int kCh = 16;           // tokens per staged chunk
-constexpr int kCols = 16;         // value columns per wave
+constexpr int kCols = 8;          // value columns per wave
+constexpr int kSlices = TL_WAVE / kCols;
+// the sum over the lanes c, c + 8, ..., c + 56; every lane gets it
+__device__ __forceinline__ float sum_over_slices(float v) { return sum_over_rows(v + dpp_f32<TL_DPP_ROR8>(v)); }
 template <int DS>
 __global__ __launch_bounds__(TL_WAVE) void delta_recurrence_kernel(
     const float* __restrict__ qn, const float* __restrict__ kn, const float* __restrict__ vc,
     const float* __restrict__ beta, const float* __restrict__ decay, float* __restrict__ state, int64_t state_stride,
     const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ state_slots, float* __restrict__ out,
     int heads, int dim, int vdim) {
-  constexpr int DP = 4 * DS;                      // key channels, padded
+  constexpr int DP = kSlices * DS;                // key channels, padded
   constexpr int PER = kCh * DP / TL_WAVE;         // floats of one staged array a lane moves per chunk
   __shared__ float ks[kCh][DP], qs[kCh][DP], gs[kCh][DP], vs[kCh][kCols], bs[kCh];
   const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
@@ -183,7 +186,7 @@ __global__ __launch_bounds__(TL_WAVE) void delta_recurrence_kernel(
         S[i] *= g[i];
         sk = fmaf(S[i], k[i], sk);
       }
-      sk = sum_over_rows(sk);
+      sk = sum_over_slices(sk);
       const float u = bs[tt] * (vs[tt][c] - sk);
       float o = 0.f;
 #pragma unroll
@@ -191,7 +194,7 @@ __global__ __launch_bounds__(TL_WAVE) void delta_recurrence_kernel(
         S[i] = fmaf(k[i], u, S[i]);
         o = fmaf(S[i], q[i], o);
       }
-      o = sum_over_rows(o);
+      o = sum_over_slices(o);
       if (s == 0 && live) out[((int64_t)(tc + tt) * heads + h) * vdim + col] = o;
     }
   }
@@ -231,15 +234,23 @@ __device__ __forceinline__ float block_sum_dyn(float v, float* red, int nw) {
 // A decode step in one kernel: every request brings ONE token.  One workgroup per (request, head),
 // a thread per value column: the convolutions, unit vectors, decay and beta of the token, the
 // recurrence on the column in registers, and the head's norm and gate on the way out
-// (z[t, h, :] = w * o / rms(o) * sigmoid(gate)).  The saved convolution inputs are read here and
-// brought up to date by conv_state_update_kernel behind it.
+// (z[t, h, :] = w * o / rms(o) * sigmoid(gate)).  The saved convolution inputs are brought up to date
+// here when every head has q/k channels of its own (update_saved); else several workgroups read a
+// channel's saved inputs and conv_state_update_kernel runs behind this kernel.
+constexpr int kDecodeThreads = 256;     // value columns the one-kernel decode step takes (a thread each)
+template <typename T>
+__device__ __forceinline__ void shift_saved(const T* __restrict__ p, int64_t p_stride, int t, int col,
+                                            float* __restrict__ saved, int taps) {
+  for (int i = 0; i + 2 < taps; ++i) saved[i] = saved[i + 1];
+  if (taps > 1) saved[taps - 2] = to_f32(p[(int64_t)t * p_stride + col]);
+}
 template <typename T, int DIM>
-__global__ void delta_decode_kernel(
+__global__ __launch_bounds__(kDecodeThreads) void delta_decode_kernel(
     const T* __restrict__ p, int64_t p_stride, int conv_off, int b_off, const float* __restrict__ low, int64_t low_stride,
     const float* __restrict__ conv_w, const float* __restrict__ a_log, const float* __restrict__ dt_bias,
     const float* __restrict__ w_norm, float* __restrict__ state, int64_t state_stride, int64_t saved_off,
     const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ state_slots, T* __restrict__ z, int heads,
-    int kv_heads, int dim, int vdim, int taps, float q_scale, float eps) {
+    int kv_heads, int dim, int vdim, int taps, float q_scale, float eps, int update_saved) {
   __shared__ float qs[kMaxDim], ks[kMaxDim], gs[kMaxDim], red[16];
   const int r = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
   const int nw = blockDim.x / TL_WAVE;
@@ -247,7 +258,7 @@ __global__ void delta_decode_kernel(
   if (cu_seqlens[r + 1] - t != 1) return;         // a padding request owns no state
   const int kh = h / (heads / kv_heads);
   float* row = state + (int64_t)state_slots[r] * state_stride;
-  const float* saved = row + saved_off;
+  float* saved = row + saved_off;
   const int q_ch = kh * dim, k_ch = kv_heads * dim + kh * dim, v_ch = 2 * kv_heads * dim + h * vdim;
   float sq = 0.f, sk = 0.f;
   const float rate = expf(a_log[h]);
@@ -256,6 +267,10 @@ __global__ void delta_decode_kernel(
                               conv_w + (int64_t)(q_ch + i) * taps, taps);
     const float k = conv_silu(p, p_stride, t, 0, conv_off + k_ch + i, saved + (int64_t)(k_ch + i) * (taps - 1),
                               conv_w + (int64_t)(k_ch + i) * taps, taps);
+    if (update_saved) {         // no other head reads these channels: this thread is their only reader
+      shift_saved(p, p_stride, t, conv_off + q_ch + i, saved + (int64_t)(q_ch + i) * (taps - 1), taps);
+      shift_saved(p, p_stride, t, conv_off + k_ch + i, saved + (int64_t)(k_ch + i) * (taps - 1), taps);
+    }
     qs[i] = q;
     ks[i] = k;
     sq += q * q;
@@ -270,6 +285,7 @@ __global__ void delta_decode_kernel(
   if (col < vdim) {
     const float v = conv_silu(p, p_stride, t, 0, conv_off + v_ch + col, saved + (int64_t)(v_ch + col) * (taps - 1),
                               conv_w + (int64_t)(v_ch + col) * taps, taps);
+    if (update_saved) shift_saved(p, p_stride, t, conv_off + v_ch + col, saved + (int64_t)(v_ch + col) * (taps - 1), taps);
     const float beta = 1.f / (1.f + expf(-to_f32(p[(int64_t)t * p_stride + b_off + h])));
     float* S_mem = row + (int64_t)h * dim * vdim + col;
     float S[DIM];
@@ -348,11 +364,11 @@ int tl_delta_recurrence(const float* qn, const float* kn, const float* vc, const
 #define TL_REC(DS)                                                                                                   \
   hipLaunchKernelGGL(delta_recurrence_kernel<DS>, g, b, 0, stream, qn, kn, vc, beta, decay, state, state_stride,     \
                      cu_seqlens, state_slots, out, heads, dim, vdim)
-  if (dim <= 16) TL_REC(4);
-  else if (dim <= 32) TL_REC(8);
-  else if (dim <= 64) TL_REC(16);
-  else if (dim <= 128) TL_REC(32);
-  else TL_REC(64);
+  if (dim <= 16) TL_REC(2);
+  else if (dim <= 32) TL_REC(4);
+  else if (dim <= 64) TL_REC(8);
+  else if (dim <= 128) TL_REC(16);
+  else TL_REC(32);
 #undef TL_REC
   return tl_launch_status();
 }
@@ -362,16 +378,16 @@ int tl_delta_decode(const void* p, int64_t p_stride, int conv_off, int b_off, co
                     const float* conv_w, const float* a_log, const float* dt_bias, const float* w_norm, float* state,
                     int64_t state_stride, int64_t saved_off, const int32_t* cu_seqlens, const int32_t* state_slots,
                     void* z, int n_requests, int heads, int kv_heads, int dim, int vdim, int taps, float q_scale,
-                    float eps, int dtype, hipStream_t stream) {
+                    float eps, int update_saved, int dtype, hipStream_t stream) {
   if (n_requests <= 0) return TL_OK;
   if (heads <= 0 || heads > 65535 || kv_heads <= 0 || heads % kv_heads || dim <= 0 || dim > kMaxDim || vdim <= 0 ||
-      vdim > 1024 || taps < 1 || taps > kMaxTaps)
+      vdim > kDecodeThreads || taps < 1 || taps > kMaxTaps || (update_saved && heads != kv_heads))
     return TL_ERR_ARG;
   dim3 g(n_requests, heads), b((vdim + TL_WAVE - 1) / TL_WAVE * TL_WAVE);
 #define TL_DEC(TT, D)                                                                                               \
   hipLaunchKernelGGL((delta_decode_kernel<TT, D>), g, b, 0, stream, (const TT*)p, p_stride, conv_off, b_off, low,   \
                      low_stride, conv_w, a_log, dt_bias, w_norm, state, state_stride, saved_off, cu_seqlens,        \
-                     state_slots, (TT*)z, heads, kv_heads, dim, vdim, taps, q_scale, eps)
+                     state_slots, (TT*)z, heads, kv_heads, dim, vdim, taps, q_scale, eps, update_saved)
 #define TL_DEC_D(TT)                  \
   if (dim <= 16) TL_DEC(TT, 16);      \
   else if (dim <= 32) TL_DEC(TT, 32); \

@@ -352,8 +352,10 @@ __global__ __launch_bounds__(LF_WAVES * TL_WAVE) void latent_flash_bf16_kernel(
     }
 }
 
-// Merges the partial results of `n_splits` workgroups: one wave per (token, head); maxima are in
-// units of log2 e; a split without keys has l = 0.
+// Merges the partial results of `n_splits` (<= 64) workgroups: one wave per (token, head).  Lane s
+// fetches split s's maximum and sum, the weights 2^(m_s - M) are formed once, and the output dims are
+// then summed over the splits with every load independent of the others.  Maxima are in units of
+// log2 e; a split without keys has l = 0.
 __global__ __launch_bounds__(TL_WAVE) void latent_combine_kernel(const float* __restrict__ part,
                                                                  const bf16_t* __restrict__ gate, int64_t gate_stride,
                                                                  bf16_t* __restrict__ out, int n_tokens, int heads,
@@ -361,52 +363,83 @@ __global__ __launch_bounds__(TL_WAVE) void latent_combine_kernel(const float* __
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int MROW = kv_rank + 2;
   const int64_t row = (int64_t)t * heads + h, step = (int64_t)n_tokens * heads;
-  float M = kNegBig;
-  for (int s = 0; s < n_splits; ++s) M = fmaxf(M, part[(row + s * step) * MROW + kv_rank]);
-  float L = 0.f;
-  for (int s = 0; s < n_splits; ++s)
-    L += __builtin_amdgcn_exp2f(part[(row + s * step) * MROW + kv_rank] - M) * part[(row + s * step) * MROW + kv_rank + 1];
+  const bool mine = lane < n_splits;
+  const float m = mine ? part[(row + lane * step) * MROW + kv_rank] : kNegBig;
+  const float l = mine ? part[(row + lane * step) * MROW + kv_rank + 1] : 0.f;
+  const float M = wave_max(m);
+  const float wgt = mine ? __builtin_amdgcn_exp2f(m - M) : 0.f;
+  const float L = wave_sum(wgt * l);
   float f = L > 0.f ? 1.f / L : 0.f;
   if (gate) f /= 1.f + expf(-(float)gate[(int64_t)t * gate_stride + h]);
-  for (int d = lane; d < kv_rank; d += TL_WAVE) {
-    float acc = 0.f;
-    for (int s = 0; s < n_splits; ++s)
-      acc += __builtin_amdgcn_exp2f(part[(row + s * step) * MROW + kv_rank] - M) * part[(row + s * step) * MROW + d];
-    out[row * kv_rank + d] = (bf16_t)(acc * f);
+  float acc[kRPL];
+#pragma unroll
+  for (int i = 0; i < kRPL; ++i) acc[i] = 0.f;
+  for (int s = 0; s < n_splits; ++s) {
+    const float ws = __shfl(wgt, s, TL_WAVE);
+    const float* src = part + (row + s * step) * MROW;
+#pragma unroll
+    for (int i = 0; i < kRPL; ++i) {
+      const int d = lane + i * TL_WAVE;
+      if (d < kv_rank) acc[i] = fmaf(ws, src[d], acc[i]);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < kRPL; ++i) {
+    const int d = lane + i * TL_WAVE;
+    if (d < kv_rank) out[row * kv_rank + d] = (bf16_t)(acc[i] * f);
   }
 }
 
 // Small products per head for steps of few rows: out[t, h, n] = sum_k w[h, k, n] * in[t, h, k].
-// The weights lie [heads, inner, cols], so that the threads of a workgroup (one per output column)
-// read them in whole lines; a workgroup takes up to kRows rows at a time, whose inputs it keeps in LDS.
+// The weights lie [heads, inner, cols].  A workgroup owns 32 output columns of one head for up to kRows
+// rows: its eight groups of 32 threads take every eighth k each (a group reads 64 contiguous bytes of a
+// weight row, sixteen rows requested at a time), and the eight partial sums meet in LDS in a fixed order.
 constexpr int kRows = 8;
 constexpr int kMaxInner = 1024;
+constexpr int kHpCols = 32, kHpSlices = kThreads / kHpCols;
 template <typename TI, typename TW, typename TO>
 __global__ __launch_bounds__(kThreads) void head_products_kernel(const TI* __restrict__ in, int64_t in_stride,
                                                                  int in_head_width, const TW* __restrict__ w,
                                                                  TO* __restrict__ out, int64_t out_stride,
                                                                  int out_head_width, int n_rows, int inner, int cols) {
   __shared__ float xs[kRows][kMaxInner];
-  const int h = blockIdx.x, n = blockIdx.y * kThreads + threadIdx.x;
+  __shared__ float part[kHpSlices][kRows][kHpCols];
+  const int h = blockIdx.x, cn = threadIdx.x % kHpCols, sl = threadIdx.x / kHpCols;
+  const int n = blockIdx.y * kHpCols + cn;
   const int t0 = blockIdx.z * kRows, rows = min(kRows, n_rows - t0);
-  for (int e = threadIdx.x; e < rows * inner; e += kThreads) {
+  for (int e = threadIdx.x; e < kRows * inner; e += kThreads) {
     const int r = e / inner, k = e - r * inner;
-    xs[r][k] = to_f32(in[(int64_t)(t0 + r) * in_stride + (int64_t)h * in_head_width + k]);
+    xs[r][k] = r < rows ? to_f32(in[(int64_t)(t0 + r) * in_stride + (int64_t)h * in_head_width + k]) : 0.f;
   }
   __syncthreads();
-  if (n >= cols) return;
   float acc[kRows];
 #pragma unroll
   for (int r = 0; r < kRows; ++r) acc[r] = 0.f;
-  const TW* wp = w + (int64_t)h * inner * cols + n;
-  for (int k = 0; k < inner; ++k) {
-    const float wv = to_f32(wp[(int64_t)k * cols]);
+  const TW* wp = w + (int64_t)h * inner * cols + min(n, cols - 1);
+  for (int k0 = sl; k0 < inner; k0 += kHpSlices * 16) {
+    float wv[16];
 #pragma unroll
-    for (int r = 0; r < kRows; ++r) acc[r] = fmaf(wv, xs[r][k], acc[r]);      // rows beyond `rows` hold stale LDS: never stored
+    for (int u = 0; u < 16; ++u) {
+      const int k = k0 + u * kHpSlices;
+      wv[u] = k < inner ? to_f32(wp[(int64_t)k * cols]) : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+      const int k = min(k0 + u * kHpSlices, inner - 1);
+#pragma unroll
+      for (int r = 0; r < kRows; ++r) acc[r] = fmaf(wv[u], xs[r][k], acc[r]);
+    }
   }
 #pragma unroll
-  for (int r = 0; r < kRows; ++r)
-    if (r < rows) out[(int64_t)(t0 + r) * out_stride + (int64_t)h * out_head_width + n] = from_f32<TO>(acc[r]);
+  for (int r = 0; r < kRows; ++r) part[sl][r][cn] = acc[r];
+  __syncthreads();
+  for (int e = threadIdx.x; e < rows * kHpCols; e += kThreads) {
+    const int r = e / kHpCols, c2 = e % kHpCols, n2 = blockIdx.y * kHpCols + c2;
+    float sum = 0.f;
+#pragma unroll
+    for (int q = 0; q < kHpSlices; ++q) sum += part[q][r][c2];
+    if (n2 < cols) out[(int64_t)(t0 + r) * out_stride + (int64_t)h * out_head_width + n2] = from_f32<TO>(sum);
+  }
 }
 
 }  // namespace
@@ -472,7 +505,7 @@ int tl_latent_flash(const float* qa, const void* latent, const void* rope, const
                     int n_splits, hipStream_t stream) {
   if (n_tiles <= 0 || n_tokens <= 0) return TL_OK;
   if (heads <= 0 || kv_rank <= 0 || kv_rank % 16 || kv_rank > 16 * LF_MAXDT || rot < 0 || rot % 8 ||
-      kv_rank + rot > 32 * LF_MAXKS || block_size <= 0 || max_blocks <= 0 || n_splits < 1 || n_splits > 65535 ||
+      kv_rank + rot > 32 * LF_MAXKS || block_size <= 0 || max_blocks <= 0 || n_splits < 1 || n_splits > TL_WAVE ||
       tpt != 16 / (heads < 16 ? heads : 16) || (n_splits > 1 && !part) || (heads + 15) / 16 > 65535)
     return TL_ERR_ARG;
   const int WP = (kv_rank + rot + 31) / 32 * 32;
@@ -501,9 +534,9 @@ int tl_head_products(const void* in, int64_t in_stride, int in_head_width, const
                      int out_dtype, hipStream_t stream) {
   if (n_rows <= 0) return TL_OK;
   if (heads <= 0 || inner <= 0 || inner > kMaxInner || cols <= 0 || inner > in_head_width || cols > out_head_width ||
-      (n_rows + kRows - 1) / kRows > 65535 || (cols + kThreads - 1) / kThreads > 65535)
+      (n_rows + kRows - 1) / kRows > 65535 || (cols + kHpCols - 1) / kHpCols > 65535)
     return TL_ERR_ARG;
-  dim3 g(heads, (cols + kThreads - 1) / kThreads, (n_rows + kRows - 1) / kRows), b(kThreads);
+  dim3 g(heads, (cols + kHpCols - 1) / kHpCols, (n_rows + kRows - 1) / kRows), b(kThreads);
 #define TL_HP(TI, TO)                                                                                              \
   hipLaunchKernelGGL((head_products_kernel<TI, TI, TO>), g, b, 0, stream, (const TI*)in, in_stride, in_head_width, \
                      (const TI*)w, (TO*)out, out_stride, out_head_width, n_rows, inner, cols)

@@ -12,14 +12,43 @@ constexpr int kWaves = kThreads / TL_WAVE;
 
 // x[t] += scale * w * y[t] / sqrt(mean(y[t]^2) + eps); copy[t] = x[t] in TC (optional).
 // One workgroup per row.  `w` is the norm's effective weight, `scale` (optional) a factor per channel.
+// Rows of up to kKeep * kThreads elements stay in registers between the two passes, and what the second
+// pass needs (x, w, scale) is requested before the sum of squares is known.
+constexpr int kKeep = 8;
 template <typename TC>
-__global__ void norm_scale_add_kernel(const float* __restrict__ y, const float* __restrict__ w,
-                                      const float* __restrict__ scale, float* __restrict__ x,
-                                      TC* __restrict__ copy, int hidden, float eps) {
+__global__ __launch_bounds__(kThreads) void norm_scale_add_kernel(const float* __restrict__ y,
+                                                                  const float* __restrict__ w,
+                                                                  const float* __restrict__ scale,
+                                                                  float* __restrict__ x, TC* __restrict__ copy,
+                                                                  int hidden, float eps) {
   __shared__ float red[kWaves];
   const float* src = y + (int64_t)blockIdx.x * hidden;
   float* dst = x + (int64_t)blockIdx.x * hidden;
   float ss = 0.f;
+  if (hidden <= kKeep * kThreads) {
+    float yv[kKeep], xv[kKeep], wv[kKeep];
+#pragma unroll
+    for (int i = 0; i < kKeep; ++i) {
+      const int j = threadIdx.x + i * kThreads;
+      const bool in = j < hidden;
+      yv[i] = in ? src[j] : 0.f;
+      xv[i] = in ? dst[j] : 0.f;
+      wv[i] = in ? (scale ? w[j] * scale[j] : w[j]) : 0.f;
+      ss += yv[i] * yv[i];
+    }
+    ss = block_sum<kWaves>(ss, red);
+    const float r = 1.f / sqrtf(ss / (float)hidden + eps);
+#pragma unroll
+    for (int i = 0; i < kKeep; ++i) {
+      const int j = threadIdx.x + i * kThreads;
+      if (j < hidden) {
+        const float s = xv[i] + yv[i] * r * wv[i];
+        dst[j] = s;
+        if (copy) copy[(int64_t)blockIdx.x * hidden + j] = from_f32<TC>(s);
+      }
+    }
+    return;
+  }
   for (int j = threadIdx.x; j < hidden; j += kThreads) {
     const float v = src[j];
     ss += v * v;

@@ -1400,17 +1400,18 @@ def delta_recurrence(qn: torch.Tensor, kn: torch.Tensor, vc: torch.Tensor, beta:
     return out
 
 
-DELTA_DECODE_MAX_VDIM = 1024     # a thread per value column in the one-kernel decode step
+DELTA_DECODE_MAX_VDIM = 256      # a thread per value column in the one-kernel decode step
 
 
 def delta_decode(p: torch.Tensor, conv_off: int, b_off: int, low: torch.Tensor, conv_w: torch.Tensor,
                  a_log: torch.Tensor, dt_bias: torch.Tensor, w_norm: torch.Tensor, state: torch.Tensor,
                  saved_off: int, cu_seqlens: torch.Tensor, state_slots: torch.Tensor, z: torch.Tensor, heads: int,
-                 kv_heads: int, dim: int, vdim: int, taps: int, q_scale: float, eps: float) -> torch.Tensor:
+                 kv_heads: int, dim: int, vdim: int, taps: int, q_scale: float, eps: float) -> bool:
     """A decode step of the delta rule in one kernel (every request brings one token; row t of the
     operands is request t): what `delta_prepare`, `delta_recurrence` and `head_norm_gate` do, with
-    `low` [T, heads * dim + heads * vdim] float32 = [decay | gate] pre-activations.  The saved
-    convolution inputs are read only: `conv_state_update` follows."""
+    `low` [T, heads * dim + heads * vdim] float32 = [decay | gate] pre-activations.  Returns whether
+    the saved convolution inputs were brought up to date as well (every head has q/k channels of its
+    own); if not, `conv_state_update` has to follow."""
     _dev(p, low, conv_w, a_log, dt_bias, w_norm, state, cu_seqlens, state_slots, z)
     check_delta_sizes(heads, kv_heads, dim, vdim, taps)
     _rows_2d(p, "projections")
@@ -1433,9 +1434,10 @@ def delta_decode(p: torch.Tensor, conv_off: int, b_off: int, low: torch.Tensor, 
                                   c_int64(low.stride(0)), _ptr(conv_w), _ptr(a_log), _ptr(dt_bias), _ptr(w_norm),
                                   _ptr(state), c_int64(state.stride(0)), c_int64(saved_off), _ptr(cu_seqlens),
                                   _ptr(state_slots), _ptr(z), c_int(R), c_int(heads), c_int(kv_heads), c_int(dim),
-                                  c_int(vdim), c_int(taps), c_float(q_scale), c_float(eps), c_int(_dt(p)), _stream()),
+                                  c_int(vdim), c_int(taps), c_float(q_scale), c_float(eps), c_int(heads == kv_heads),
+                                  c_int(_dt(p)), _stream()),
            "delta_decode")
-    return z
+    return heads == kv_heads
 
 
 def head_norm_gate(o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, out: torch.Tensor, heads: int,

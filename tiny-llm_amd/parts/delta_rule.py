@@ -111,11 +111,12 @@ class ChannelDelta(Mixer):
         z = ops.scratch("delta_gated", (T, H * V), self.dtype, dev)
         if ctx.max_q_len == 1 and T == ctx.num_requests and V <= ops.DELTA_DECODE_MAX_VDIM:
             # decoding: every request brings one token; convolutions, recurrence, norm and gate in one kernel
-            ops.delta_decode(p, 0, self.b_off, low, self.conv_w, self.a_log, self.dt_bias, self.w_norm, state,
-                             self.state_size, ctx.cu_seqlens_q, ctx.state_slots, z, H, KH, D, V, self.taps, D ** -0.5,
-                             self.eps)
-            ops.conv_state_update(p, 0, self.channels, state, self.state_size, ctx.cu_seqlens_q, ctx.state_slots,
-                                  self.taps)
+            saved = ops.delta_decode(p, 0, self.b_off, low, self.conv_w, self.a_log, self.dt_bias, self.w_norm, state,
+                                     self.state_size, ctx.cu_seqlens_q, ctx.state_slots, z, H, KH, D, V, self.taps,
+                                     D ** -0.5, self.eps)
+            if not saved:       # heads share q/k channels: their saved inputs are shifted behind the kernel
+                ops.conv_state_update(p, 0, self.channels, state, self.state_size, ctx.cu_seqlens_q,
+                                      ctx.state_slots, self.taps)
             return self._project_out(z, residual)
         qn = ops.scratch("delta_q", (T * H * D,), torch.float32, dev)
         kn = ops.scratch("delta_k", (T * H * D,), torch.float32, dev)
