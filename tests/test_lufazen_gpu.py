@@ -383,3 +383,19 @@ def test_head_products(dtype):
             tol = 1e-5 if out_dtype == torch.float32 else 2e-2
             assert (out[:, :, :N].double().cpu() - want).abs().max() < tol
             assert extra == 0 or torch.isnan(out[:, :, N:]).all()      # nothing is written beside the view
+
+
+def test_head_gemm():
+    """The same products for many rows on the matrix cores, with edges in every direction."""
+    from tiny_llm_amd.kernels import ops
+    g = torch.Generator().manual_seed(6)
+    for T, H, K, N, extra in ((33, 3, 24, 40, 8), (200, 2, 40, 16, 0), (70, 4, 128, 72, 16), (64, 1, 520, 33, 8)):
+        x = torch.randn(T, H, K + extra, generator=g).to(torch.bfloat16).cuda()
+        w = (torch.randn(H, N, K, generator=g) / K ** 0.5).to(torch.bfloat16).cuda()
+        want = torch.einsum("thk,hnk->thn", x[:, :, :K].double().cpu(), w.double().cpu())
+        for out_dtype in (torch.bfloat16, torch.float32):
+            out = torch.full((T, H, N + extra), float("nan"), dtype=out_dtype, device="cuda")
+            ops.head_gemm(x[:, :, :K], w, out[:, :, :N])
+            tol = 1e-4 if out_dtype == torch.float32 else 2e-2
+            assert (out[:, :, :N].double().cpu() - want).abs().max() < tol
+            assert extra == 0 or torch.isnan(out[:, :, N:]).all()

@@ -442,6 +442,62 @@ __global__ __launch_bounds__(kThreads) void head_products_kernel(const TI* __res
   }
 }
 
+// The same products for steps of many rows, on the matrix cores (bfloat16): out[t, h, n] =
+// sum_k w[h, n, k] * in[t, h, k] with the weights [heads, cols, inner] (k contiguous, as the checkpoint
+// stores them).  A workgroup of four waves owns 64 columns x 64 rows of one head, a wave 32 x 32 as
+// 2 x 2 tiles of v_mfma_f32_16x16x32_bf16; both operands go straight from memory into registers (a
+// lane's eight consecutive k of one row).  The product is computed transposed (columns as the
+// instruction's rows), so a lane ends with four consecutive output columns of one row.
+template <typename TO>
+__global__ __launch_bounds__(kThreads) void head_gemm_bf16_kernel(const bf16_t* __restrict__ in, int64_t in_stride,
+                                                                  int in_head_width, const bf16_t* __restrict__ w,
+                                                                  TO* __restrict__ out, int64_t out_stride,
+                                                                  int out_head_width, int n_rows, int inner, int cols) {
+  const int h = blockIdx.x, wave = threadIdx.x / TL_WAVE, lane = threadIdx.x % TL_WAVE, g = lane / 16, c = lane % 16;
+  const int col0 = blockIdx.y * 64 + (wave & 1) * 32, row0 = blockIdx.z * 64 + (wave >> 1) * 32;
+  if (col0 >= cols || row0 >= n_rows) return;
+  const bf16_t* wp[2];
+  const bf16_t* xp[2];
+#pragma unroll
+  for (int a = 0; a < 2; ++a) {
+    wp[a] = w + ((int64_t)h * cols + min(col0 + a * 16 + c, cols - 1)) * inner;
+    xp[a] = in + (int64_t)min(row0 + a * 16 + c, n_rows - 1) * in_stride + (int64_t)h * in_head_width;
+  }
+  f32x4 acc[2][2];
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int b = 0; b < 2; ++b) acc[a][b] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  for (int k0 = 0; k0 < inner; k0 += 32) {
+    const int d0 = k0 + g * 8;
+    bf16x8 wa[2], xb[2];
+#pragma unroll
+    for (int a = 0; a < 2; ++a) {
+      wa[a] = d0 < inner ? *(const bf16x8*)(wp[a] + d0) : zero;
+      xb[a] = d0 < inner ? *(const bf16x8*)(xp[a] + d0) : zero;
+    }
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+      for (int b = 0; b < 2; ++b) acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[a], xb[b], acc[a][b], 0, 0, 0);
+  }
+  // acc[a][b][i] = out[row0 + b*16 + c][col0 + a*16 + g*4 + i]
+#pragma unroll
+  for (int b = 0; b < 2; ++b) {
+    const int row = row0 + b * 16 + c;
+    if (row >= n_rows) continue;
+#pragma unroll
+    for (int a = 0; a < 2; ++a) {
+      const int n = col0 + a * 16 + g * 4;
+      TO* dst = out + (int64_t)row * out_stride + (int64_t)h * out_head_width + n;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (n + i < cols) dst[i] = from_f32<TO>(acc[a][b][i]);
+    }
+  }
+}
+
 }  // namespace
 
 #define TL_DISPATCH_T(dtype, ...)                 \
@@ -545,6 +601,25 @@ int tl_head_products(const void* in, int64_t in_stride, int in_head_width, const
   else if (dtype == 1 && out_dtype == 1) TL_HP(bf16_t, bf16_t);
   else return TL_ERR_ARG;
 #undef TL_HP
+  return tl_launch_status();
+}
+
+// bfloat16, many rows: w [heads, cols, inner]; inner a multiple of 8, operands 16-byte aligned.
+int tl_head_gemm(const void* in, int64_t in_stride, int in_head_width, const void* w, void* out, int64_t out_stride,
+                 int out_head_width, int n_rows, int heads, int inner, int cols, int out_dtype, hipStream_t stream) {
+  if (n_rows <= 0) return TL_OK;
+  if (heads <= 0 || inner <= 0 || inner % 8 || cols <= 0 || inner > in_head_width || cols > out_head_width ||
+      in_stride % 8 || in_head_width % 8 || (n_rows + 63) / 64 > 65535 || (cols + 63) / 64 > 65535)
+    return TL_ERR_ARG;
+  dim3 g(heads, (cols + 63) / 64, (n_rows + 63) / 64), b(kThreads);
+  if (out_dtype == 0)
+    hipLaunchKernelGGL(head_gemm_bf16_kernel<float>, g, b, 0, stream, (const bf16_t*)in, in_stride, in_head_width,
+                       (const bf16_t*)w, (float*)out, out_stride, out_head_width, n_rows, inner, cols);
+  else if (out_dtype == 1)
+    hipLaunchKernelGGL(head_gemm_bf16_kernel<bf16_t>, g, b, 0, stream, (const bf16_t*)in, in_stride, in_head_width,
+                       (const bf16_t*)w, (bf16_t*)out, out_stride, out_head_width, n_rows, inner, cols);
+  else
+    return TL_ERR_ARG;
   return tl_launch_status();
 }
 

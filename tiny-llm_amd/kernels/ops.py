@@ -1312,6 +1312,24 @@ def head_products(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.
     return out
 
 
+def head_gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[t, h, :] = w[h] x[t, h, :] for every head in one launch on the matrix cores (bfloat16, any
+    number of rows): x [T, heads, inner] and out [T, heads, cols] may be views into wider rows; w
+    [heads, cols, inner] contiguous; out bfloat16 or float32."""
+    _dev(x, w, out)
+    T, H = x.shape[0], x.shape[1]
+    cols, inner = w.shape[1], w.shape[2]
+    if not (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.dim() == 3 and out.dim() == 3 and w.dim() == 3
+            and w.is_contiguous() and w.shape[0] == H and x.stride(2) == 1 and out.stride(2) == 1
+            and tuple(out.shape[:2]) == (T, H) and x.shape[2] == inner and out.shape[2] == cols and inner % 8 == 0
+            and x.stride(0) % 8 == 0 and x.stride(1) % 8 == 0 and out.dtype in (torch.bfloat16, torch.float32)):
+        _fail("head_gemm: bfloat16 x [T, heads, inner] (inner and strides multiples of 8), w [heads, cols, inner], out [T, heads, cols]")
+    _check(_lib().tl_head_gemm(_ptr(x, 16), c_int64(x.stride(0)), c_int(x.stride(1)), _ptr(w, 16), _ptr(out),
+                               c_int64(out.stride(0)), c_int(out.stride(1)), c_int(T), c_int(H), c_int(inner),
+                               c_int(cols), c_int(_dt(out)), _stream()), "head_gemm")
+    return out
+
+
 # ------------------------------------------------------------------ gated delta rule
 DELTA_MAX_DIM = 256     # key channels of a head (csrc/delta_rule.hip)
 DELTA_MAX_TAPS = 16

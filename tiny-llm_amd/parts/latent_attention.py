@@ -139,8 +139,11 @@ class LatentAttention(Mixer):
         qa = ops.scratch("latent_qa", (T, H, KR + R), torch.float32, dev)
         q3, qa2 = q.view(T, H, D + R), qa.view(T, H * (KR + R))
         few = T <= ops.HEAD_PRODUCT_ROWS and max(D, KR) <= ops.HEAD_PRODUCT_INNER
+        many = self.dtype == torch.bfloat16 and not few          # one launch on the matrix cores
         if few:
             ops.head_products(q3[:, :, :D], self.w_uk_few, qa[:, :, :KR])
+        elif many:
+            ops.head_gemm(q3[:, :, :D], self.w_uk_t, qa[:, :, :KR])
         else:
             for n in range(H):
                 ops.linear(q3[:, n, :D], self.w_uk_t[n], qa2[:, n * (KR + R):n * (KR + R) + KR])
@@ -166,6 +169,8 @@ class LatentAttention(Mixer):
         o = ops.scratch("latent_heads", (T, H * V), self.dtype, dev)
         if few:
             ops.head_products(mix, self.w_uv_few, o.view(T, H, V))
+        elif many:
+            ops.head_gemm(mix, self.w_uv.view(H, V, KR), o.view(T, H, V))
         else:
             for n in range(H):
                 ops.linear(mix[:, n, :], self.w_uv[n * V:(n + 1) * V], o[:, n * V:(n + 1) * V])
