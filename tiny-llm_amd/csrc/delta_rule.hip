@@ -27,11 +27,24 @@ __device__ __forceinline__ float conv_input(const T* __restrict__ p, int64_t p_s
   return m >= 0 ? to_f32(p[(int64_t)(t0 + m) * p_stride + col]) : saved[(taps - 1) + m];
 }
 
+// Up to four taps (the usual sizes) are requested together; the sum runs from the oldest input to the
+// current one either way.
 template <typename T>
 __device__ __forceinline__ float conv_silu(const T* __restrict__ p, int64_t p_stride, int t0, int n, int col,
                                            const float* __restrict__ saved, const float* __restrict__ w, int taps) {
   float acc = 0.f;
-  for (int b = 0; b < taps; ++b) acc = fmaf(w[taps - 1 - b], conv_input(p, p_stride, t0, n - b, col, saved, taps), acc);
+  if (taps <= 4) {
+    float x[4], wt[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {       // tap j of the weights meets input n - (taps - 1) + j
+      x[j] = j < taps ? conv_input(p, p_stride, t0, n - (taps - 1) + j, col, saved, taps) : 0.f;
+      wt[j] = j < taps ? w[j] : 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc = fmaf(wt[j], x[j], acc);
+    return silu(acc);
+  }
+  for (int j = 0; j < taps; ++j) acc = fmaf(w[j], conv_input(p, p_stride, t0, n - (taps - 1) + j, col, saved, taps), acc);
   return silu(acc);
 }
 
@@ -238,20 +251,43 @@ __device__ __forceinline__ float block_sum_dyn(float v, float* red, int nw) {
 // here when every head has q/k channels of its own (update_saved); else several workgroups read a
 // channel's saved inputs and conv_state_update_kernel runs behind this kernel.
 constexpr int kDecodeThreads = 256;     // value columns the one-kernel decode step takes (a thread each)
+// The inputs and weights of one channel's convolution for the token at row t (n = 0 in its step),
+// oldest first; taps <= 4.
 template <typename T>
-__device__ __forceinline__ void shift_saved(const T* __restrict__ p, int64_t p_stride, int t, int col,
-                                            float* __restrict__ saved, int taps) {
-  for (int i = 0; i + 2 < taps; ++i) saved[i] = saved[i + 1];
-  if (taps > 1) saved[taps - 2] = to_f32(p[(int64_t)t * p_stride + col]);
+__device__ __forceinline__ void load_taps(const T* __restrict__ p, int64_t p_stride, int t, int col,
+                                          const float* __restrict__ saved, const float* __restrict__ w, int taps,
+                                          float* x, float* wt) {
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    x[j] = j < taps ? conv_input(p, p_stride, t, j - (taps - 1), col, saved, taps) : 0.f;
+    wt[j] = j < taps ? w[j] : 0.f;
+  }
 }
-template <typename T, int DIM>
+__device__ __forceinline__ float conv_of(const float* x, const float* wt) {
+  float acc = 0.f;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) acc = fmaf(wt[j], x[j], acc);
+  return silu(acc);
+}
+// after the token the saved inputs are the last taps - 1 of x
+__device__ __forceinline__ void store_saved(float* __restrict__ saved, const float* x, int taps) {
+#pragma unroll
+  for (int j = 1; j < 4; ++j)
+    if (j < taps) saved[j - 1] = x[j];
+}
+
+// State phase of the kernel: thread (sl, cq) keeps rows [sl * DS, (sl + 1) * DS) of the FOUR value columns
+// 4 cq .. 4 cq + 3 of S in registers (16-byte loads and stores: a lane that moves four bytes at a time gets a
+// fraction of what a compute unit can fetch), the four slices' partial sums meet in LDS in a fixed order.
+template <typename T, int DS>
 __global__ __launch_bounds__(kDecodeThreads) void delta_decode_kernel(
     const T* __restrict__ p, int64_t p_stride, int conv_off, int b_off, const float* __restrict__ low, int64_t low_stride,
     const float* __restrict__ conv_w, const float* __restrict__ a_log, const float* __restrict__ dt_bias,
     const float* __restrict__ w_norm, float* __restrict__ state, int64_t state_stride, int64_t saved_off,
     const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ state_slots, T* __restrict__ z, int heads,
     int kv_heads, int dim, int vdim, int taps, float q_scale, float eps, int update_saved) {
-  __shared__ float qs[kMaxDim], ks[kMaxDim], gs[kMaxDim], red[16];
+  __shared__ float qs[kMaxDim], ks[kMaxDim], gs[kMaxDim], vs[kDecodeThreads], red[16];
+  __shared__ f32x4 part[4][kDecodeThreads / 4];
   const int r = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
   const int nw = blockDim.x / TL_WAVE;
   const int t = cu_seqlens[r];
@@ -260,58 +296,111 @@ __global__ __launch_bounds__(kDecodeThreads) void delta_decode_kernel(
   float* row = state + (int64_t)state_slots[r] * state_stride;
   float* saved = row + saved_off;
   const int q_ch = kh * dim, k_ch = kv_heads * dim + kh * dim, v_ch = 2 * kv_heads * dim + h * vdim;
-  float sq = 0.f, sk = 0.f;
+  const int quads = vdim / 4;
+  const int cq = tid % quads, sl = tid / quads;     // state phase: column quad and slice of the key channels
+  const bool owner = sl < 4;
+  // Everything the token needs is requested here, before the first value is used.
+  float xq[4], wq[4], xk[4], wk[4], xv[4], wv[4];
+  const int i0 = min(tid, dim - 1), c0 = min(tid, vdim - 1);        // threads beyond read what exists
+  float* sv_q = saved + (int64_t)(q_ch + i0) * (taps - 1);
+  float* sv_k = saved + (int64_t)(k_ch + i0) * (taps - 1);
+  float* sv_v = saved + (int64_t)(v_ch + c0) * (taps - 1);
+  load_taps(p, p_stride, t, conv_off + q_ch + i0, sv_q, conv_w + (int64_t)(q_ch + i0) * taps, taps, xq, wq);
+  load_taps(p, p_stride, t, conv_off + k_ch + i0, sv_k, conv_w + (int64_t)(k_ch + i0) * taps, taps, xk, wk);
+  load_taps(p, p_stride, t, conv_off + v_ch + c0, sv_v, conv_w + (int64_t)(v_ch + c0) * taps, taps, xv, wv);
+  const float pre_a = low[(int64_t)t * low_stride + h * dim + i0] + dt_bias[h * dim + i0];
+  const float pre_b = to_f32(p[(int64_t)t * p_stride + b_off + h]);
   const float rate = expf(a_log[h]);
-  for (int i = tid; i < dim; i += blockDim.x) {
-    const float q = conv_silu(p, p_stride, t, 0, conv_off + q_ch + i, saved + (int64_t)(q_ch + i) * (taps - 1),
-                              conv_w + (int64_t)(q_ch + i) * taps, taps);
-    const float k = conv_silu(p, p_stride, t, 0, conv_off + k_ch + i, saved + (int64_t)(k_ch + i) * (taps - 1),
-                              conv_w + (int64_t)(k_ch + i) * taps, taps);
+  float pre_g[4], wn[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    pre_g[e] = low[(int64_t)t * low_stride + heads * dim + h * vdim + cq * 4 + e];
+    wn[e] = w_norm[cq * 4 + e];
+  }
+  float* S_mem = row + (int64_t)h * dim * vdim + cq * 4;
+  f32x4 S[DS];
+#pragma unroll
+  for (int j = 0; j < DS; ++j) {
+    const int i = sl * DS + j;
+    S[j] = (owner && i < dim) ? *(const f32x4*)(S_mem + (int64_t)i * vdim) : f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  float sq = 0.f, sk = 0.f;
+  if (tid < dim) {
+    const float q = conv_of(xq, wq), k = conv_of(xk, wk);
+    qs[tid] = q;
+    ks[tid] = k;
+    sq = q * q;
+    sk = k * k;
+    gs[tid] = expf(-rate * softplus(pre_a));
     if (update_saved) {         // no other head reads these channels: this thread is their only reader
-      shift_saved(p, p_stride, t, conv_off + q_ch + i, saved + (int64_t)(q_ch + i) * (taps - 1), taps);
-      shift_saved(p, p_stride, t, conv_off + k_ch + i, saved + (int64_t)(k_ch + i) * (taps - 1), taps);
+      store_saved(sv_q, xq, taps);
+      store_saved(sv_k, xk, taps);
     }
-    qs[i] = q;
-    ks[i] = k;
-    sq += q * q;
-    sk += k * k;
-    gs[i] = expf(-rate * softplus(low[(int64_t)t * low_stride + h * dim + i] + dt_bias[h * dim + i]));
+  }
+  if (tid < vdim) {
+    vs[tid] = conv_of(xv, wv);
+    if (update_saved) store_saved(sv_v, xv, taps);
   }
   sq = block_sum_dyn(sq, red, nw);
-  sk = block_sum_dyn(sk, red, nw);      // its barriers also make qs, ks and gs visible
+  sk = block_sum_dyn(sk, red, nw);      // its barriers also make qs, ks, gs and vs visible
   const float rq = q_scale / sqrtf(sq + 1e-6f), rk = 1.f / sqrtf(sk + 1e-6f);
-  const int col = tid;
-  float o = 0.f;
-  if (col < vdim) {
-    const float v = conv_silu(p, p_stride, t, 0, conv_off + v_ch + col, saved + (int64_t)(v_ch + col) * (taps - 1),
-                              conv_w + (int64_t)(v_ch + col) * taps, taps);
-    if (update_saved) shift_saved(p, p_stride, t, conv_off + v_ch + col, saved + (int64_t)(v_ch + col) * (taps - 1), taps);
-    const float beta = 1.f / (1.f + expf(-to_f32(p[(int64_t)t * p_stride + b_off + h])));
-    float* S_mem = row + (int64_t)h * dim * vdim + col;
-    float S[DIM];
+  const float beta = 1.f / (1.f + expf(-pre_b));
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  if (owner) {
 #pragma unroll
-    for (int i = 0; i < DIM; ++i) S[i] = i < dim ? S_mem[(int64_t)i * vdim] : 0.f;
-    float acc = 0.f;
-#pragma unroll
-    for (int i = 0; i < DIM; ++i)
+    for (int j = 0; j < DS; ++j) {
+      const int i = sl * DS + j;
       if (i < dim) {
-        S[i] *= gs[i];
-        acc = fmaf(S[i], ks[i] * rk, acc);
-      }
-    const float u = beta * (v - acc);
+        const float g = gs[i], k = ks[i] * rk;
 #pragma unroll
-    for (int i = 0; i < DIM; ++i)
-      if (i < dim) {
-        S[i] = fmaf(ks[i] * rk, u, S[i]);
-        o = fmaf(S[i], qs[i] * rq, o);
-        S_mem[(int64_t)i * vdim] = S[i];
+        for (int e = 0; e < 4; ++e) {
+          S[j][e] *= g;
+          acc[e] = fmaf(S[j][e], k, acc[e]);
+        }
       }
+    }
+    part[sl][cq] = acc;
   }
-  const float ss = block_sum_dyn(col < vdim ? o * o : 0.f, red, nw);
-  if (col < vdim) {
-    const float g = low[(int64_t)t * low_stride + heads * dim + h * vdim + col];
-    z[((int64_t)t * heads + h) * vdim + col] =
-        from_f32<T>(o / sqrtf(ss / (float)vdim + eps) * w_norm[col] / (1.f + expf(-g)));
+  __syncthreads();
+  f32x4 o = {0.f, 0.f, 0.f, 0.f};
+  if (owner) {
+    const f32x4 p0 = part[0][cq], p1 = part[1][cq], p2 = part[2][cq], p3 = part[3][cq];
+    f32x4 u;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) u[e] = beta * (vs[cq * 4 + e] - (((p0[e] + p1[e]) + p2[e]) + p3[e]));
+#pragma unroll
+    for (int j = 0; j < DS; ++j) {
+      const int i = sl * DS + j;
+      if (i < dim) {
+        const float k = ks[i] * rk, q = qs[i] * rq;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          S[j][e] = fmaf(k, u[e], S[j][e]);
+          o[e] = fmaf(S[j][e], q, o[e]);
+        }
+        *(f32x4*)(S_mem + (int64_t)i * vdim) = S[j];
+      }
+    }
+  }
+  __syncthreads();                      // the first round's sums have been read
+  if (owner) part[sl][cq] = o;
+  __syncthreads();
+  float oo = 0.f;
+  if (sl == 0) {
+    const f32x4 p0 = part[0][cq], p1 = part[1][cq], p2 = part[2][cq], p3 = part[3][cq];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      o[e] = ((p0[e] + p1[e]) + p2[e]) + p3[e];
+      oo += o[e] * o[e];
+    }
+  }
+  const float ss = block_sum_dyn(oo, red, nw);
+  if (sl == 0) {
+    const float rn = 1.f / sqrtf(ss / (float)vdim + eps);
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      z[((int64_t)t * heads + h) * vdim + cq * 4 + e] = from_f32<T>(o[e] * rn * wn[e] / (1.f + expf(-pre_g[e])));
   }
 }
 
@@ -381,19 +470,21 @@ int tl_delta_decode(const void* p, int64_t p_stride, int conv_off, int b_off, co
                     float eps, int update_saved, int dtype, hipStream_t stream) {
   if (n_requests <= 0) return TL_OK;
   if (heads <= 0 || heads > 65535 || kv_heads <= 0 || heads % kv_heads || dim <= 0 || dim > kMaxDim || vdim <= 0 ||
-      vdim > kDecodeThreads || taps < 1 || taps > kMaxTaps || (update_saved && heads != kv_heads))
+      vdim > kDecodeThreads || vdim % 4 || state_stride % 4 || dim > kDecodeThreads || taps < 1 || taps > 4 ||
+      (update_saved && heads != kv_heads))
     return TL_ERR_ARG;
-  dim3 g(n_requests, heads), b((vdim + TL_WAVE - 1) / TL_WAVE * TL_WAVE);
+  const int threads = vdim > dim ? vdim : dim;      // a thread per value column and per key channel
+  dim3 g(n_requests, heads), b((threads + TL_WAVE - 1) / TL_WAVE * TL_WAVE);
 #define TL_DEC(TT, D)                                                                                               \
   hipLaunchKernelGGL((delta_decode_kernel<TT, D>), g, b, 0, stream, (const TT*)p, p_stride, conv_off, b_off, low,   \
                      low_stride, conv_w, a_log, dt_bias, w_norm, state, state_stride, saved_off, cu_seqlens,        \
                      state_slots, (TT*)z, heads, kv_heads, dim, vdim, taps, q_scale, eps, update_saved)
 #define TL_DEC_D(TT)                  \
-  if (dim <= 16) TL_DEC(TT, 16);      \
-  else if (dim <= 32) TL_DEC(TT, 32); \
-  else if (dim <= 64) TL_DEC(TT, 64); \
-  else if (dim <= 128) TL_DEC(TT, 128); \
-  else TL_DEC(TT, 256);
+  if (dim <= 16) TL_DEC(TT, 4);       \
+  else if (dim <= 32) TL_DEC(TT, 8);  \
+  else if (dim <= 64) TL_DEC(TT, 16); \
+  else if (dim <= 128) TL_DEC(TT, 32); \
+  else TL_DEC(TT, 64);
   if (dtype == 0) { TL_DEC_D(float) }
   else if (dtype == 1) { TL_DEC_D(bf16_t) }
   else return TL_ERR_ARG;

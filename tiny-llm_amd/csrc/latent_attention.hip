@@ -203,15 +203,34 @@ __global__ __launch_bounds__(LF_WAVES * TL_WAVE) void latent_flash_bf16_kernel(
   bf16_t* Vl = Qlo + 16 * QS + wave * 16 * VS;
   const int32_t* bt = block_tables + (int64_t)r * max_blocks;
 
-  // the query tile as q = hi + lo in bfloat16; rows without a query and dims beyond W are zero
-  for (int e = threadIdx.x; e < 16 * WP; e += LF_WAVES * TL_WAVE) {
-    const int row = e / WP, d = e - row * WP;
-    const int tt = row / hg, h = head0 + row % hg;
-    float v = 0.f;
-    if (tt < ntok && tt < tpt && h < heads && d < W) v = qa[((int64_t)(tok0 + tt) * heads + h) * W + d];
-    const bf16_t hi = (bf16_t)v;
-    Ql[row * QS + d] = hi;
-    Qlo[row * QS + d] = (bf16_t)(v - (float)hi);
+  // the query tile as q = hi + lo in bfloat16; rows without a query and dims beyond W are zero.  Sixteen
+  // threads a row, four consecutive floats at a time, everything requested before anything is used.
+  {
+    const int qrow = threadIdx.x / 16, seg = threadIdx.x % 16;
+    const int tt = qrow / hg, hh = head0 + qrow % hg;
+    const bool has = tt < ntok && tt < tpt && hh < heads;
+    const float* qsrc = qa + ((int64_t)(tok0 + min(tt, ntok - 1)) * heads + min(hh, heads - 1)) * W;
+    constexpr int NQ = LF_MAXKS / 2;                  // 64 floats a step of the sixteen threads
+    f32x4 qv[NQ];
+#pragma unroll
+    for (int j = 0; j < NQ; ++j) {
+      const int d = seg * 4 + 64 * j;
+      qv[j] = (has && d < W) ? *(const f32x4*)(qsrc + d) : f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+#pragma unroll
+    for (int j = 0; j < NQ; ++j) {
+      const int d = seg * 4 + 64 * j;
+      if (d < WP) {
+        bf16x4 hi, lo;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          hi[i] = (bf16_t)qv[j][i];
+          lo[i] = (bf16_t)(qv[j][i] - (float)hi[i]);
+        }
+        *(bf16x4*)(Ql + qrow * QS + d) = hi;
+        *(bf16x4*)(Qlo + qrow * QS + d) = lo;
+      }
+    }
   }
   const int my_tt = c / hg, my_h = head0 + c % hg;
   const bool row_valid = my_tt < ntok && my_tt < tpt && my_h < heads;
@@ -374,14 +393,23 @@ __global__ __launch_bounds__(TL_WAVE) void latent_combine_kernel(const float* __
   float acc[kRPL];
 #pragma unroll
   for (int i = 0; i < kRPL; ++i) acc[i] = 0.f;
-  for (int s = 0; s < n_splits; ++s) {
-    const float ws = __shfl(wgt, s, TL_WAVE);
-    const float* src = part + (row + s * step) * MROW;
+  for (int s0 = 0; s0 < n_splits; s0 += 4) {         // four splits requested at a time
+    float v[4][kRPL], ws[4];
 #pragma unroll
-    for (int i = 0; i < kRPL; ++i) {
-      const int d = lane + i * TL_WAVE;
-      if (d < kv_rank) acc[i] = fmaf(ws, src[d], acc[i]);
+    for (int u = 0; u < 4; ++u) {
+      const int s = min(s0 + u, n_splits - 1);
+      ws[u] = s0 + u < n_splits ? __shfl(wgt, s, TL_WAVE) : 0.f;
+      const float* src = part + (row + s * step) * MROW;
+#pragma unroll
+      for (int i = 0; i < kRPL; ++i) {
+        const int d = lane + i * TL_WAVE;
+        v[u][i] = d < kv_rank ? src[d] : 0.f;
+      }
     }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int i = 0; i < kRPL; ++i) acc[i] = fmaf(ws[u], v[u][i], acc[i]);
   }
 #pragma unroll
   for (int i = 0; i < kRPL; ++i) {
@@ -407,9 +435,19 @@ __global__ __launch_bounds__(kThreads) void head_products_kernel(const TI* __res
   const int h = blockIdx.x, cn = threadIdx.x % kHpCols, sl = threadIdx.x / kHpCols;
   const int n = blockIdx.y * kHpCols + cn;
   const int t0 = blockIdx.z * kRows, rows = min(kRows, n_rows - t0);
-  for (int e = threadIdx.x; e < kRows * inner; e += kThreads) {
-    const int r = e / inner, k = e - r * inner;
-    xs[r][k] = r < rows ? to_f32(in[(int64_t)(t0 + r) * in_stride + (int64_t)h * in_head_width + k]) : 0.f;
+  {                                   // the rows' inputs: everything requested before anything is stored
+    constexpr int NX = kRows * kMaxInner / kThreads;
+    float tmp[NX];
+#pragma unroll
+    for (int j = 0; j < NX; ++j) {
+      const int e = threadIdx.x + j * kThreads, r = e / inner, k = e - r * inner;
+      tmp[j] = (e < kRows * inner && r < rows) ? to_f32(in[(int64_t)(t0 + r) * in_stride + (int64_t)h * in_head_width + k]) : 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < NX; ++j) {
+      const int e = threadIdx.x + j * kThreads, r = e / inner, k = e - r * inner;
+      if (e < kRows * inner) xs[r][k] = tmp[j];
+    }
   }
   __syncthreads();
   float acc[kRows];

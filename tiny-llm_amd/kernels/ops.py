@@ -1419,6 +1419,7 @@ def delta_recurrence(qn: torch.Tensor, kn: torch.Tensor, vc: torch.Tensor, beta:
 
 
 DELTA_DECODE_MAX_VDIM = 256      # a thread per value column in the one-kernel decode step
+DELTA_DECODE_MAX_TAPS = 4         # and its convolutions' inputs in registers
 
 
 def delta_decode(p: torch.Tensor, conv_off: int, b_off: int, low: torch.Tensor, conv_w: torch.Tensor,
@@ -1443,7 +1444,8 @@ def delta_decode(p: torch.Tensor, conv_off: int, b_off: int, low: torch.Tensor, 
     _f32_vec(w_norm, vdim, "the head norm's weight")
     if not (p.shape[0] == R and low.shape[0] == R and low.dtype == torch.float32
             and low.shape[1] >= heads * (dim + vdim) and conv_off + channels <= p.shape[1] and b_off + heads <= p.shape[1]
-            and cu_seqlens.numel() == R + 1 and vdim <= DELTA_DECODE_MAX_VDIM
+            and cu_seqlens.numel() == R + 1 and vdim <= DELTA_DECODE_MAX_VDIM and taps <= DELTA_DECODE_MAX_TAPS
+            and vdim % 4 == 0 and state.stride(0) % 4 == 0
             and state.dtype == torch.float32 and state.dim() == 2 and state.is_contiguous()
             and saved_off + channels * (taps - 1) <= state.shape[1] and heads * dim * vdim <= saved_off
             and z.dtype == p.dtype and z.is_contiguous() and tuple(z.shape) == (R, heads * vdim)):

@@ -98,7 +98,8 @@ class ChannelDelta(Mixer):
         self.a_log, self.dt_bias, self.w_norm = f32(tensors[n["A_log"]]), f32(tensors[n["dt_bias"]]), f32(tensors[n["norm"]])
 
     def state_spec(self) -> StateSpec:
-        return StateSpec((self.state_size + self.channels * (self.taps - 1),), torch.float32)
+        # a multiple of four floats: rows of the state start at 16-byte boundaries
+        return StateSpec((-(-(self.state_size + self.channels * (self.taps - 1)) // 4) * 4,), torch.float32)
 
     # --------------------------------------------------------------------- compute
     def forward(self, h, ctx, cache, state, residual):
@@ -109,7 +110,8 @@ class ChannelDelta(Mixer):
         low = ops.scratch("delta_low", (T, H * D + H * V), torch.float32, dev)
         ops.linear(p[:, self.low_off:self.low_off + self.ra + self.rg], self.w_low, low)
         z = ops.scratch("delta_gated", (T, H * V), self.dtype, dev)
-        if ctx.max_q_len == 1 and T == ctx.num_requests and V <= ops.DELTA_DECODE_MAX_VDIM:
+        if ctx.max_q_len == 1 and T == ctx.num_requests and V <= ops.DELTA_DECODE_MAX_VDIM and V % 4 == 0 \
+                and self.taps <= ops.DELTA_DECODE_MAX_TAPS:
             # decoding: every request brings one token; convolutions, recurrence, norm and gate in one kernel
             saved = ops.delta_decode(p, 0, self.b_off, low, self.conv_w, self.a_log, self.dt_bias, self.w_norm, state,
                                      self.state_size, ctx.cu_seqlens_q, ctx.state_slots, z, H, KH, D, V, self.taps,
