@@ -379,7 +379,7 @@ def test_head_products(dtype):
         want = torch.einsum("thk,hkn->thn", x[:, :, :K].double().cpu(), w.double().cpu())
         for out_dtype in {dtype, torch.float32}:
             out = torch.full((T, H, N + extra), float("nan"), dtype=out_dtype, device="cuda")
-            ops.head_products(x[:, :, :K], w, out[:, :, :N])
+            ops.head_products(x[:, :, :K], ops.head_product_weights(w), out[:, :, :N])
             tol = 1e-5 if out_dtype == torch.float32 else 2e-2
             assert (out[:, :, :N].double().cpu() - want).abs().max() < tol
             assert extra == 0 or torch.isnan(out[:, :, N:]).all()      # nothing is written beside the view

@@ -419,21 +419,39 @@ __global__ __launch_bounds__(TL_WAVE) void latent_combine_kernel(const float* __
 }
 
 // Small products per head for steps of few rows: out[t, h, n] = sum_k w[h, k, n] * in[t, h, k].
-// The weights lie [heads, inner, cols].  A workgroup owns 32 output columns of one head for up to kRows
-// rows: its eight groups of 32 threads take every eighth k each (a group reads 64 contiguous bytes of a
-// weight row, sixteen rows requested at a time), and the eight partial sums meet in LDS in a fixed order.
+// The weights lie [heads, inner, cols_padded] (cols_padded a multiple of 8).  A workgroup owns 64 output
+// columns of one head for up to kRows rows.  A lane is (k slice, column octet): it fetches eight columns
+// of one weight row in one access and takes every 32nd k (eight slices a wave, four waves); the eight
+// slices of a wave meet through lane exchanges, the four waves in LDS, both in a fixed order.
 constexpr int kRows = 8;
 constexpr int kMaxInner = 1024;
-constexpr int kHpCols = 32, kHpSlices = kThreads / kHpCols;
+constexpr int kHpCols = 64, kHpSlices = 32;
+template <typename TW>
+__device__ __forceinline__ void load8(const TW* p, float* v) {
+  if constexpr (sizeof(TW) == 2) {
+    const bf16x8 x = *(const bf16x8*)p;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = (float)x[e];
+  } else {
+    const f32x4 a = *(const f32x4*)p, b2 = *(const f32x4*)(p + 4);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      v[e] = a[e];
+      v[4 + e] = b2[e];
+    }
+  }
+}
 template <typename TI, typename TW, typename TO>
 __global__ __launch_bounds__(kThreads) void head_products_kernel(const TI* __restrict__ in, int64_t in_stride,
                                                                  int in_head_width, const TW* __restrict__ w,
                                                                  TO* __restrict__ out, int64_t out_stride,
-                                                                 int out_head_width, int n_rows, int inner, int cols) {
+                                                                 int out_head_width, int n_rows, int inner, int cols,
+                                                                 int cols_padded) {
   __shared__ float xs[kRows][kMaxInner];
-  __shared__ float part[kHpSlices][kRows][kHpCols];
-  const int h = blockIdx.x, cn = threadIdx.x % kHpCols, sl = threadIdx.x / kHpCols;
-  const int n = blockIdx.y * kHpCols + cn;
+  __shared__ float part[kWaves][kRows][kHpCols];
+  const int h = blockIdx.x, wave = threadIdx.x / TL_WAVE, lane = threadIdx.x % TL_WAVE;
+  const int oc = lane % 8, slice = wave * 8 + lane / 8;
+  const int col0 = blockIdx.y * kHpCols;
   const int t0 = blockIdx.z * kRows, rows = min(kRows, n_rows - t0);
   {                                   // the rows' inputs: everything requested before anything is stored
     constexpr int NX = kRows * kMaxInner / kThreads;
@@ -450,32 +468,55 @@ __global__ __launch_bounds__(kThreads) void head_products_kernel(const TI* __res
     }
   }
   __syncthreads();
-  float acc[kRows];
+  float acc[kRows][8];
 #pragma unroll
-  for (int r = 0; r < kRows; ++r) acc[r] = 0.f;
-  const TW* wp = w + (int64_t)h * inner * cols + min(n, cols - 1);
-  for (int k0 = sl; k0 < inner; k0 += kHpSlices * 16) {
-    float wv[16];
+  for (int r = 0; r < kRows; ++r)
 #pragma unroll
-    for (int u = 0; u < 16; ++u) {
+    for (int e = 0; e < 8; ++e) acc[r][e] = 0.f;
+  const bool has_cols = col0 + oc * 8 < cols_padded;
+  const TW* wp = w + (int64_t)h * inner * cols_padded + min(col0 + oc * 8, cols_padded - 8);
+  for (int k0 = slice; k0 < inner; k0 += kHpSlices * 4) {        // four weight rows requested at a time
+    float wv[4][8];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
       const int k = k0 + u * kHpSlices;
-      wv[u] = k < inner ? to_f32(wp[(int64_t)k * cols]) : 0.f;
+      load8(wp + (int64_t)min(k, inner - 1) * cols_padded, wv[u]);
+      if (k >= inner || !has_cols) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) wv[u][e] = 0.f;
+      }
     }
 #pragma unroll
-    for (int u = 0; u < 16; ++u) {
+    for (int u = 0; u < 4; ++u) {
       const int k = min(k0 + u * kHpSlices, inner - 1);
 #pragma unroll
-      for (int r = 0; r < kRows; ++r) acc[r] = fmaf(wv[u], xs[r][k], acc[r]);
+      for (int r = 0; r < kRows; ++r) {
+        const float x = xs[r][k];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[r][e] = fmaf(wv[u][e], x, acc[r][e]);
+      }
     }
   }
+  // the eight slices of the wave: lanes oc, oc + 8, ..., oc + 56
 #pragma unroll
-  for (int r = 0; r < kRows; ++r) part[sl][r][cn] = acc[r];
+  for (int r = 0; r < kRows; ++r)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float v = acc[r][e];
+      acc[r][e] = sum_over_rows(v + dpp_f32<TL_DPP_ROR8>(v));
+    }
+  if (lane < 8) {
+#pragma unroll
+    for (int r = 0; r < kRows; ++r)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) part[wave][r][oc * 8 + e] = acc[r][e];
+  }
   __syncthreads();
   for (int e = threadIdx.x; e < rows * kHpCols; e += kThreads) {
-    const int r = e / kHpCols, c2 = e % kHpCols, n2 = blockIdx.y * kHpCols + c2;
+    const int r = e / kHpCols, c2 = e % kHpCols, n2 = col0 + c2;
     float sum = 0.f;
 #pragma unroll
-    for (int q = 0; q < kHpSlices; ++q) sum += part[q][r][c2];
+    for (int q = 0; q < kWaves; ++q) sum += part[q][r][c2];
     if (n2 < cols) out[(int64_t)(t0 + r) * out_stride + (int64_t)h * out_head_width + n2] = from_f32<TO>(sum);
   }
 }
@@ -621,19 +662,20 @@ int tl_latent_flash(const float* qa, const void* latent, const void* rope, const
   return tl_launch_status();
 }
 
-// in / out: rows with a stride, head h at column h * head_width.  w [heads, inner, cols] of in's type;
+// in / out: rows with a stride, head h at column h * head_width.  w [heads, inner, cols_padded] of in's type;
 // out float32 (out_dtype 0) or of in's type.
 int tl_head_products(const void* in, int64_t in_stride, int in_head_width, const void* w, void* out,
-                     int64_t out_stride, int out_head_width, int n_rows, int heads, int inner, int cols, int dtype,
-                     int out_dtype, hipStream_t stream) {
+                     int64_t out_stride, int out_head_width, int n_rows, int heads, int inner, int cols,
+                     int cols_padded, int dtype, int out_dtype, hipStream_t stream) {
   if (n_rows <= 0) return TL_OK;
   if (heads <= 0 || inner <= 0 || inner > kMaxInner || cols <= 0 || inner > in_head_width || cols > out_head_width ||
+      cols_padded < cols || cols_padded % 8 ||
       (n_rows + kRows - 1) / kRows > 65535 || (cols + kHpCols - 1) / kHpCols > 65535)
     return TL_ERR_ARG;
   dim3 g(heads, (cols + kHpCols - 1) / kHpCols, (n_rows + kRows - 1) / kRows), b(kThreads);
 #define TL_HP(TI, TO)                                                                                              \
   hipLaunchKernelGGL((head_products_kernel<TI, TI, TO>), g, b, 0, stream, (const TI*)in, in_stride, in_head_width, \
-                     (const TI*)w, (TO*)out, out_stride, out_head_width, n_rows, inner, cols)
+                     (const TI*)w, (TO*)out, out_stride, out_head_width, n_rows, inner, cols, cols_padded)
   if (dtype == 0 && out_dtype == 0) TL_HP(float, float);
   else if (dtype == 1 && out_dtype == 0) TL_HP(bf16_t, float);
   else if (dtype == 1 && out_dtype == 1) TL_HP(bf16_t, bf16_t);

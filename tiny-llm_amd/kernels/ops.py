@@ -1294,21 +1294,30 @@ HEAD_PRODUCT_ROWS = 32      # up to this many rows the per-head products of a st
 HEAD_PRODUCT_INNER = 1024
 
 
+def head_product_weights(w: torch.Tensor) -> torch.Tensor:
+    """w [heads, inner, cols] as `head_products` wants it: contiguous, the columns padded with zeros to
+    a multiple of 8 (a lane fetches eight columns of a weight row at once)."""
+    pad = -w.shape[2] % 8
+    return torch.nn.functional.pad(w, (0, pad)).contiguous() if pad else w.contiguous()
+
+
 def head_products(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     """out[t, h, :] = w[h]^T x[t, h, :] for every head in one launch (steps of few rows):
     x [T, heads, >= inner] and out [T, heads, >= cols] may be views into wider rows (any row and
-    head stride, unit inner stride); w [heads, inner, cols] contiguous of x's type; out float32 or x's type."""
+    head stride, unit inner stride); w [heads, inner, cols rounded up to 8] from `head_product_weights`,
+    of x's type; out float32 or x's type (its last size says how many columns are real)."""
     _dev(x, w, out)
     T, H = x.shape[0], x.shape[1]
-    inner, cols = w.shape[1], w.shape[2]
+    inner, cols = w.shape[1], out.shape[2]
     if not (x.dim() == 3 and out.dim() == 3 and w.dim() == 3 and w.is_contiguous() and w.shape[0] == H
             and w.dtype == x.dtype and x.stride(2) == 1 and out.stride(2) == 1 and tuple(out.shape[:2]) == (T, H)
-            and x.shape[2] == inner and out.shape[2] == cols and inner <= HEAD_PRODUCT_INNER
-            and (out.dtype == x.dtype or out.dtype == torch.float32)):
-        _fail("head_products: x [T, heads, inner], w [heads, inner, cols], out [T, heads, cols]")
-    _check(_lib().tl_head_products(_ptr(x), c_int64(x.stride(0)), c_int(x.stride(1)), _ptr(w), _ptr(out),
+            and x.shape[2] == inner and w.shape[2] % 8 == 0 and 0 <= w.shape[2] - cols < 8
+            and inner <= HEAD_PRODUCT_INNER and (out.dtype == x.dtype or out.dtype == torch.float32)):
+        _fail("head_products: x [T, heads, inner], w [heads, inner, cols rounded up to 8], out [T, heads, cols]")
+    _check(_lib().tl_head_products(_ptr(x), c_int64(x.stride(0)), c_int(x.stride(1)), _ptr(w, 16), _ptr(out),
                                    c_int64(out.stride(0)), c_int(out.stride(1)), c_int(T), c_int(H), c_int(inner),
-                                   c_int(cols), c_int(_dt(x)), c_int(_dt(out)), _stream()), "head_products")
+                                   c_int(cols), c_int(w.shape[2]), c_int(_dt(x)), c_int(_dt(out)), _stream()),
+           "head_products")
     return out
 
 

@@ -104,8 +104,8 @@ class LatentAttention(Mixer):
         self.w_uk_t = uk.transpose(1, 2).contiguous()
         self.w_uv = tensors[n["uv"]].contiguous()
         # the same two as [heads, inner, cols], for the one-launch products of steps with few rows
-        self.w_uk_few = uk.contiguous()
-        self.w_uv_few = self.w_uv.view(H, self.value_dim, self.kv_rank).transpose(1, 2).contiguous()
+        self.w_uk_few = ops.head_product_weights(uk)
+        self.w_uv_few = ops.head_product_weights(self.w_uv.view(H, self.value_dim, self.kv_rank).transpose(1, 2))
         self.w_o = tensors[n["o"]].contiguous()
 
     def cache_spec(self) -> CacheSpec:
