@@ -123,28 +123,31 @@ __global__ void conv_state_update_kernel(const T* __restrict__ p, int64_t p_stri
     if (i < taps - 1) saved[i] = next[i];
 }
 
-// The recurrence.  One wave per (request, head, 8 value columns): lane (s, c) keeps rows
+// The recurrence.  A wave owns 8 value columns of one (request, head): lane (s, c) keeps rows
 // [s * DS, (s + 1) * DS) of column c of S in registers (eight slices of the key channels side by side,
 // 8 lanes each), so a token costs DS steps and two sums over the eight slices instead of `dim` steps.
 // The wave walks the request's tokens of this step in order, kCh at a time: q, k, decay, v and beta of a
-// chunk go through LDS, and the next chunk's are requested before this one is worked on.
+// chunk go through LDS, and the next chunk's are requested before this one is worked on.  The four waves
+// of a workgroup (32 columns) share the staged chunk: q, k and decay are the same for every column.
 constexpr int kCh = 16;           // tokens per staged chunk
 constexpr int kCols = 8;          // value columns per wave
+constexpr int kRecWaves = 4, kRecThreads = kRecWaves * TL_WAVE, kRecCols = kRecWaves * kCols;
 constexpr int kSlices = TL_WAVE / kCols;
 // the sum over the lanes c, c + 8, ..., c + 56; every lane gets it
 __device__ __forceinline__ float sum_over_slices(float v) { return sum_over_rows(v + dpp_f32<TL_DPP_ROR8>(v)); }
 template <int DS>
-__global__ __launch_bounds__(TL_WAVE) void delta_recurrence_kernel(
+__global__ __launch_bounds__(kRecThreads) void delta_recurrence_kernel(
     const float* __restrict__ qn, const float* __restrict__ kn, const float* __restrict__ vc,
     const float* __restrict__ beta, const float* __restrict__ decay, float* __restrict__ state, int64_t state_stride,
     const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ state_slots, float* __restrict__ out,
     int heads, int dim, int vdim) {
   constexpr int DP = kSlices * DS;                // key channels, padded
-  constexpr int PER = kCh * DP / TL_WAVE;         // floats of one staged array a lane moves per chunk
-  __shared__ float ks[kCh][DP], qs[kCh][DP], gs[kCh][DP], vs[kCh][kCols], bs[kCh];
-  const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-  const int s = lane / kCols, c = lane % kCols;
-  const int col = blockIdx.z * kCols + c;
+  constexpr int PER = (kCh * DP + kRecThreads - 1) / kRecThreads;    // floats of one staged array a thread moves per chunk
+  constexpr int PERV = kCh * kRecCols / kRecThreads;
+  __shared__ float ks[kCh][DP], qs[kCh][DP], gs[kCh][DP], vs[kCh][kRecCols], bs[kCh];
+  const int r = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, wave = tid / TL_WAVE, lane = tid % TL_WAVE;
+  const int s = lane / kCols, c = wave * kCols + lane % kCols;
+  const int col = blockIdx.z * kRecCols + c;
   const int t0 = cu_seqlens[r], t1 = cu_seqlens[r + 1];
   if (t1 <= t0) return;                           // a padding request owns no state
   const bool live = col < vdim;
@@ -153,62 +156,82 @@ __global__ __launch_bounds__(TL_WAVE) void delta_recurrence_kernel(
 #pragma unroll
   for (int i = 0; i < DS; ++i) S[i] = (live && s * DS + i < dim) ? S_mem[(int64_t)(s * DS + i) * vdim] : 0.f;
 
-  float rk[PER], rq[PER], rg[PER], rv[(kCh * kCols) / TL_WAVE], rb = 0.f;
+  float rk[PER], rq[PER], rg[PER], rv[PERV], rb = 0.f;
   // element e of a staged array: token e / DP of the chunk, channel e % DP (channels beyond dim: k = q = 0, g = 1)
   auto fetch = [&](int tc) {
 #pragma unroll
     for (int j = 0; j < PER; ++j) {
-      const int e = j * TL_WAVE + lane, tt = e / DP, i = e % DP;
-      const bool ok = tc + tt < t1 && i < dim;
+      const int e = j * kRecThreads + tid, tt = e / DP, i = e % DP;
+      const bool ok = e < kCh * DP && tc + tt < t1 && i < dim;
       const int64_t at = ((int64_t)(tc + tt) * heads + h) * dim + i;
       rk[j] = ok ? kn[at] : 0.f;
       rq[j] = ok ? qn[at] : 0.f;
       rg[j] = ok ? decay[at] : 1.f;
     }
 #pragma unroll
-    for (int j = 0; j < (kCh * kCols) / TL_WAVE; ++j) {
-      const int e = j * TL_WAVE + lane, tt = e / kCols, cc = e % kCols;
-      const int vcol = blockIdx.z * kCols + cc;
+    for (int j = 0; j < PERV; ++j) {
+      const int e = j * kRecThreads + tid, tt = e / kRecCols, cc = e % kRecCols;
+      const int vcol = blockIdx.z * kRecCols + cc;
       rv[j] = (tc + tt < t1 && vcol < vdim) ? vc[((int64_t)(tc + tt) * heads + h) * vdim + vcol] : 0.f;
     }
-    rb = (lane < kCh && tc + lane < t1) ? beta[(int64_t)(tc + lane) * heads + h] : 0.f;
+    rb = (tid < kCh && tc + tid < t1) ? beta[(int64_t)(tc + tid) * heads + h] : 0.f;
   };
   fetch(t0);
   for (int tc = t0; tc < t1; tc += kCh) {
     __syncthreads();                              // the chunk before has been read
 #pragma unroll
     for (int j = 0; j < PER; ++j) {
-      const int e = j * TL_WAVE + lane;
-      (&ks[0][0])[e] = rk[j];
-      (&qs[0][0])[e] = rq[j];
-      (&gs[0][0])[e] = rg[j];
+      const int e = j * kRecThreads + tid;
+      if (e < kCh * DP) {
+        (&ks[0][0])[e] = rk[j];
+        (&qs[0][0])[e] = rq[j];
+        (&gs[0][0])[e] = rg[j];
+      }
     }
 #pragma unroll
-    for (int j = 0; j < (kCh * kCols) / TL_WAVE; ++j) (&vs[0][0])[j * TL_WAVE + lane] = rv[j];
-    if (lane < kCh) bs[lane] = rb;
+    for (int j = 0; j < PERV; ++j) (&vs[0][0])[j * kRecThreads + tid] = rv[j];
+    if (tid < kCh) bs[tid] = rb;
     __syncthreads();
     if (tc + kCh < t1) fetch(tc + kCh);           // on its way while this chunk is worked on
     const int n = min(kCh, t1 - tc);
-    for (int tt = 0; tt < n; ++tt) {
-      const float* k = &ks[tt][s * DS];
-      const float* q = &qs[tt][s * DS];
-      const float* g = &gs[tt][s * DS];
-      float sk = 0.f;
+    // With S' = diag(g) S:  o = (S' + k u^T)^T q = S'^T q + u (k . q).  Both sums over S' and k . q are
+    // taken in ONE pass (in four independent parts) and meet in one round of exchanges between the
+    // slices; the update of S hangs off it.  A token's operands are read from LDS while the token before
+    // it is worked on (two register sets, the loop goes two tokens at a time).
+    auto load = [&](int tt, float* k, float* q, float* g, float& v, float& bt) {
+#pragma unroll
+      for (int i = 0; i < DS; ++i) {
+        k[i] = ks[tt][s * DS + i];
+        q[i] = qs[tt][s * DS + i];
+        g[i] = gs[tt][s * DS + i];
+      }
+      v = vs[tt][c];
+      bt = bs[tt];
+    };
+    auto step = [&](int tt, const float* k, const float* q, const float* g, float v, float bt) {
+      float sk[4] = {0.f, 0.f, 0.f, 0.f}, sq[4] = {0.f, 0.f, 0.f, 0.f}, kq[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int i = 0; i < DS; ++i) {
         S[i] *= g[i];
-        sk = fmaf(S[i], k[i], sk);
+        sk[i & 3] = fmaf(S[i], k[i], sk[i & 3]);
+        sq[i & 3] = fmaf(S[i], q[i], sq[i & 3]);
+        kq[i & 3] = fmaf(k[i], q[i], kq[i & 3]);
       }
-      sk = sum_over_slices(sk);
-      const float u = bs[tt] * (vs[tt][c] - sk);
-      float o = 0.f;
+      const float sk_all = sum_over_slices((sk[0] + sk[1]) + (sk[2] + sk[3]));
+      const float sq_all = sum_over_slices((sq[0] + sq[1]) + (sq[2] + sq[3]));
+      const float kq_all = sum_over_slices((kq[0] + kq[1]) + (kq[2] + kq[3]));
+      const float u = bt * (v - sk_all);
 #pragma unroll
-      for (int i = 0; i < DS; ++i) {
-        S[i] = fmaf(k[i], u, S[i]);
-        o = fmaf(S[i], q[i], o);
-      }
-      o = sum_over_slices(o);
-      if (s == 0 && live) out[((int64_t)(tc + tt) * heads + h) * vdim + col] = o;
+      for (int i = 0; i < DS; ++i) S[i] = fmaf(k[i], u, S[i]);
+      if (s == 0 && live) out[((int64_t)(tc + tt) * heads + h) * vdim + col] = fmaf(u, kq_all, sq_all);
+    };
+    float ka[DS], qa2[DS], ga[DS], kb[DS], qb[DS], gb[DS], va, ba, vb, bb;
+    load(0, ka, qa2, ga, va, ba);
+    for (int tt = 0; tt < n; tt += 2) {
+      load(min(tt + 1, kCh - 1), kb, qb, gb, vb, bb);
+      step(tt, ka, qa2, ga, va, ba);
+      load(min(tt + 2, kCh - 1), ka, qa2, ga, va, ba);
+      if (tt + 1 < n) step(tt + 1, kb, qb, gb, vb, bb);
     }
   }
 #pragma unroll
@@ -447,9 +470,9 @@ int tl_delta_recurrence(const float* qn, const float* kn, const float* vc, const
                         float* state, int64_t state_stride, const int32_t* cu_seqlens, const int32_t* state_slots,
                         float* out, int n_requests, int heads, int dim, int vdim, hipStream_t stream) {
   if (n_requests <= 0) return TL_OK;
-  if (heads <= 0 || heads > 65535 || dim <= 0 || dim > kMaxDim || vdim <= 0 || (vdim + kCols - 1) / kCols > 65535)
+  if (heads <= 0 || heads > 65535 || dim <= 0 || dim > kMaxDim || vdim <= 0 || (vdim + kRecCols - 1) / kRecCols > 65535)
     return TL_ERR_ARG;
-  dim3 g(n_requests, heads, (vdim + kCols - 1) / kCols), b(TL_WAVE);
+  dim3 g(n_requests, heads, (vdim + kRecCols - 1) / kRecCols), b(kRecThreads);
 #define TL_REC(DS)                                                                                                   \
   hipLaunchKernelGGL(delta_recurrence_kernel<DS>, g, b, 0, stream, qn, kn, vc, beta, decay, state, state_stride,     \
                      cu_seqlens, state_slots, out, heads, dim, vdim)
