@@ -14,7 +14,7 @@ constexpr int kWaves = kThreads / TL_WAVE;
 // One workgroup per row.  `w` is the norm's effective weight, `scale` (optional) a factor per channel.
 // Rows of up to kKeep * kThreads elements stay in registers between the two passes, and what the second
 // pass needs (x, w, scale) is requested before the sum of squares is known.
-constexpr int kKeep = 8;
+constexpr int kKeep = 32;
 template <typename TC>
 __global__ __launch_bounds__(kThreads) void norm_scale_add_kernel(const float* __restrict__ y,
                                                                   const float* __restrict__ w,
