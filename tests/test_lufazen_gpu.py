@@ -399,3 +399,42 @@ def test_head_gemm():
             tol = 1e-4 if out_dtype == torch.float32 else 2e-2
             assert (out[:, :, :N].double().cpu() - want).abs().max() < tol
             assert extra == 0 or torch.isnan(out[:, :, N:]).all()
+
+
+def test_command_line_and_seeded_sampling(tmp_path_factory):
+    """bin/tiny_llm serves a Lufazen folder as it serves any other (config.json chooses the model);
+    seeded sampling through the engine does not depend on what else is in the batch."""
+    folder, cfg, w, reqs, ref, block = material("A", "float32", tmp_path_factory)
+    prompt = reqs["r2"][:12]
+    proc = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "tiny_llm"), "--model_path", folder,
+                           "--nodo_sample", "--max_new_tokens=5", "--dtype", "float32", "--ignore_eos",
+                           "--prompt_ids", ",".join(map(str, prompt))], capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    got = [int(t) for t in proc.stdout.strip().splitlines()[-1].split()]
+    seq = list(prompt)
+    for _ in range(5):
+        seq.append(int(plain.forward(cfg, w, seq)[-1].argmax()))
+    assert got == seq[len(prompt):]
+    from tiny_llm_amd import Engine, SamplingParams
+    eng = Engine(folder, dtype="float32", kv_block_size=block, max_num_seqs=4, max_num_batched_tokens=64, max_model_len=256)
+    params = SamplingParams(max_new_tokens=12, do_sample=True, temperature=0.9, top_k=40, top_p=0.95, seed=7,
+                            ignore_eos=True)
+    alone = eng.generate([prompt], params)[0]
+    among = eng.generate([reqs["r0"][:30], prompt, reqs["r1"][:7]], params)[1]
+    assert alone == among
+
+
+def test_random_weights_from_a_configuration():
+    """A configuration that names the two ranks itself runs with seeded random weights (no files), as
+    the measurements do."""
+    import copy
+    from lufazen_util import MIX_A, RANKS_A
+    from tiny_llm_amd import Engine, SamplingParams
+    cfg = copy.deepcopy(MIX_A)
+    for i, (ra, rg) in RANKS_A.items():
+        cfg["layers"][i]["mixer"].update(decay_rank=ra, gate_rank=rg)
+    eng = Engine(config=cfg, dtype="bfloat16", kv_block_size=16, max_num_seqs=2, max_num_batched_tokens=32,
+                 max_model_len=128, weights_seed=3, init_std=0.05)
+    out = eng.generate([random_tokens(20, cfg["vocab"], 1), random_tokens(3, cfg["vocab"], 2)],
+                       SamplingParams.greedy(8, ignore_eos=True))
+    assert [len(o) for o in out] == [8, 8] and all(0 <= t < cfg["vocab"] for o in out for t in o)
