@@ -219,7 +219,8 @@ def _paged(rows: torch.Tensor, table, block, n_blocks, dtype):
     return pages
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, "matrix cores", "matrix cores, split keys"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, "matrix cores", "matrix cores, split keys",
+                                   "matrix cores, many rows"])
 def test_latent_attention_finds_one_key(dtype):
     """One query per place of interest is aligned with the latent of one key (and scaled so that this
     score stands out): the result must be that key's latent.  Keys at the first positions, at both
@@ -227,6 +228,7 @@ def test_latent_attention_finds_one_key(dtype):
     the query, which the mask must hide however large its score is."""
     from tiny_llm_amd.kernels import ops
     flash = isinstance(dtype, str)
+    dtype_name = dtype if flash else ""
     splits = 3 if flash and "split" in dtype else 1
     dtype = torch.bfloat16 if flash else dtype
     g = torch.Generator().manual_seed(5)
@@ -248,7 +250,12 @@ def test_latent_attention_finds_one_key(dtype):
     positions = torch.tensor([c[0] for c in cases], dtype=torch.int32, device="cuda")
     bt = torch.tensor([table + [0] * (64 - len(table))], dtype=torch.int32, device="cuda")
     out = torch.empty(T, heads, kv_rank, dtype=dtype, device="cuda")
-    if flash:
+    if flash and "many" in dtype_name:
+        # the kernel of steps with many rows: a tile per query here, each a request of its own
+        each = torch.arange(T, dtype=torch.int32, device="cuda")
+        ops.latent_prefill(qa.cuda(), pages_l, pages_r, bt.repeat(T, 1).contiguous(),
+                           (each, each.clone(), torch.ones_like(each)), positions, out, 1.0)
+    elif flash:
         # every query a request of its own (the same pages under every row of the table), as in a decode step
         part = torch.empty(splits * T * heads * (kv_rank + 2), device="cuda") if splits > 1 else None
         ops.latent_flash(qa.cuda(), pages_l, pages_r, bt.repeat(T, 1).contiguous(), None, positions, out, 1.0, None,

@@ -371,6 +371,184 @@ __global__ __launch_bounds__(LF_WAVES * TL_WAVE) void latent_flash_bf16_kernel(
     }
 }
 
+// latent_prefill_bf16_kernel: the same function for steps with many query rows.  A workgroup owns up to
+// 4 * tpt consecutive tokens of one request, a wave the 16 rows of `tpt` of them (16 heads of one token, or
+// 16 / heads tokens), and ALL its waves walk the same tiles of 32 keys: a tile [c | kr] is fetched once by the
+// whole workgroup as whole rows, staged in LDS (two buffers, one barrier a tile) and serves four times the
+// query rows; the score product reads its key operands from there, the value product reads the same rows
+// through the transposing read.  The queries are two bfloat16 terms, the upper in registers, the lower in
+// LDS.  A wave keeps its own (max, sum, output): nothing is merged.
+constexpr int LP_KEYS = 32;         // keys a staged tile holds (two 16-key tiles of the products)
+constexpr int LP_NPF = 9;           // 16-byte pieces of a staged tile a thread fetches: 32 * 72 / 256
+__global__ __launch_bounds__(LF_WAVES * TL_WAVE) void latent_prefill_bf16_kernel(
+    const float* __restrict__ qa, const bf16_t* __restrict__ latent, const bf16_t* __restrict__ rope,
+    const int32_t* __restrict__ block_tables, int max_blocks, const int32_t* __restrict__ tile_req,
+    const int32_t* __restrict__ tile_tok0, const int32_t* __restrict__ tile_ntok,
+    const int32_t* __restrict__ positions, const bf16_t* __restrict__ gate, int64_t gate_stride,
+    bf16_t* __restrict__ out, int heads, int tpt, int kv_rank, int rot, int block_size, float scale) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lf_smem[];
+  const int tid = threadIdx.x, wave = tid / TL_WAVE, lane = tid % TL_WAVE, g = lane / 16, c = lane % 16;
+  const int tile = blockIdx.x, head0 = blockIdx.y * 16;
+  const int hg = min(heads, 16);
+  const int r = tile_req[tile], tok0 = tile_tok0[tile], ntok = tile_ntok[tile];
+  if (ntok <= 0) return;                              // a padding tile
+  const int W = kv_rank + rot, WP = (W + 31) / 32 * 32, KS = WP / 32, KDT = kv_rank / 16;
+  const int KSTR = WP + LF_PAD, CPR = WP / 8;
+  bf16_t* Kl = (bf16_t*)lf_smem;                      // two buffers of LP_KEYS rows
+  bf16_t* Qlo = Kl + 2 * LP_KEYS * KSTR + wave * 16 * KSTR;     // this wave's queries' lower terms
+  const int32_t* bt = block_tables + (int64_t)r * max_blocks;
+  const int my_tt = wave * tpt + c / hg, my_h = head0 + c % hg;
+  const bool row_valid = c / hg < tpt && my_tt < ntok && my_h < heads;
+  const int my_tok = tok0 + min(my_tt, ntok - 1);
+  const int pos = positions[my_tok];
+  const int kv_end = positions[tok0 + ntok - 1] + 1;  // what the workgroup's last token sees
+  const int wave_end = wave * tpt < ntok ? positions[tok0 + min((wave + 1) * tpt, ntok) - 1] + 1 : 0;
+  const int n_kt = (kv_end + LP_KEYS - 1) / LP_KEYS;
+  const float c_log2 = scale * 1.44269504088896f;
+
+  // this lane's pieces of its query row, q = hi + lo: the upper terms stay in registers, the lower ones
+  // wait in the wave's LDS area (the registers hold the output and the tile on its way)
+  bf16x8 qh[LF_MAXKS];
+  {
+    const float* qsrc = qa + ((int64_t)my_tok * heads + min(my_h, heads - 1)) * W;
+#pragma unroll
+    for (int ks = 0; ks < LF_MAXKS; ++ks) {
+      if (ks < KS) {
+        const int d0 = ks * 32 + g * 8;
+        const bool has = row_valid && d0 < W;
+        const f32x4 a = has ? *(const f32x4*)(qsrc + d0) : f32x4{0.f, 0.f, 0.f, 0.f};
+        const f32x4 b = has ? *(const f32x4*)(qsrc + d0 + 4) : f32x4{0.f, 0.f, 0.f, 0.f};
+        bf16x8 lo;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float v = e < 4 ? a[e] : b[e - 4];
+          qh[ks][e] = (bf16_t)v;
+          lo[e] = (bf16_t)(v - (float)qh[ks][e]);
+        }
+        *(bf16x8*)(Qlo + c * KSTR + d0) = lo;
+      }
+    }
+  }
+  // A staged tile is fetched in pieces: piece f is row f / CPR, dims 8 (f % CPR) ...  The pages of a
+  // tile are looked up an iteration before its rows are requested, so that a request never begins
+  // with a round trip of its own.
+  bf16x8 pf[LP_NPF];
+  int page[LP_NPF];
+  auto lookup = [&](int kt) {
+#pragma unroll
+    for (int j = 0; j < LP_NPF; ++j) {
+      const int f = tid + j * LF_WAVES * TL_WAVE;
+      const int key = min(kt * LP_KEYS + min(f / CPR, LP_KEYS - 1), kv_end - 1);     // keys beyond the end read a row that exists
+      page[j] = bt[key / block_size];
+    }
+  };
+  auto fetch = [&](int kt) {
+#pragma unroll
+    for (int j = 0; j < LP_NPF; ++j) {
+      const int f = tid + j * LF_WAVES * TL_WAVE;
+      if (f < LP_KEYS * CPR) {
+        const int row = f / CPR, d0 = (f - row * CPR) * 8;
+        const int key = min(kt * LP_KEYS + row, kv_end - 1);
+        const int64_t slot = (int64_t)page[j] * block_size + (key % block_size);
+        if (d0 < kv_rank) pf[j] = *(const bf16x8*)(latent + slot * kv_rank + d0);
+        else if (d0 - kv_rank < rot) pf[j] = *(const bf16x8*)(rope + slot * rot + (d0 - kv_rank));
+        else pf[j] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+      }
+    }
+  };
+  auto stage = [&](bf16_t* buf) {
+#pragma unroll
+    for (int j = 0; j < LP_NPF; ++j) {
+      const int f = tid + j * LF_WAVES * TL_WAVE;
+      if (f < LP_KEYS * CPR) {
+        const int row = f / CPR, d0 = (f - row * CPR) * 8;
+        *(bf16x8*)(buf + row * KSTR + d0) = pf[j];
+      }
+    }
+  };
+  float m_run = kNegBig, l_run = 0.f;
+  f32x4 o[LF_MAXDT];
+#pragma unroll
+  for (int dt = 0; dt < LF_MAXDT; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  lookup(0);
+  fetch(0);
+  if (n_kt > 1) lookup(1);
+  stage(Kl);
+  __syncthreads();
+  for (int kt = 0; kt < n_kt; ++kt) {
+    const bf16_t* cur = Kl + (kt & 1) * LP_KEYS * KSTR;
+    if (kt + 1 < n_kt) {
+      fetch(kt + 1);                                  // on its way while this tile is worked on
+      if (kt + 2 < n_kt) lookup(kt + 2);
+    }
+#pragma unroll
+    for (int half = 0; half < LP_KEYS / 16; ++half) {
+      const int j0 = kt * LP_KEYS + half * 16;
+      if (j0 >= wave_end) continue;                   // no key of these sixteen is seen by this wave's tokens
+      const bf16_t* rows = cur + half * 16 * KSTR;
+      f32x4 sc = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < LF_MAXKS; ++ks) {
+        if (ks < KS) {
+          const bf16x8 kop = *(const bf16x8*)(rows + c * KSTR + ks * 32 + g * 8);
+          const bf16x8 ql = *(const bf16x8*)(Qlo + c * KSTR + ks * 32 + g * 8);
+          sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop, qh[ks], sc, 0, 0, 0);
+          sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop, ql, sc, 0, 0, 0);
+        }
+      }
+      float m_tile = kNegBig;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int j = j0 + g * 4 + i;
+        const bool ok = row_valid && j <= pos;
+        sc[i] = ok ? sc[i] * c_log2 : -INFINITY;
+        m_tile = fmaxf(m_tile, sc[i]);
+      }
+      m_tile = max_over_rows(m_tile);
+      const float m_new = fmaxf(m_run, m_tile);
+      const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+      float psum = 0.f;
+      bf16x4 pb;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float p = __builtin_amdgcn_exp2f(sc[i] - m_new);
+        psum += p;
+        pb[i] = (bf16_t)p;
+      }
+      psum = sum_over_rows(psum);
+      l_run = l_run * alpha + psum;
+      m_run = m_new;
+      const bf16_t* vsrc = rows + (g * 4 + c / 4) * KSTR + 4 * (c % 4);
+#pragma unroll
+      for (int dt = 0; dt < LF_MAXDT; ++dt) {
+        if (dt < KDT) {
+          const bf16x4 vf = lf_read_transposed(vsrc + dt * 16);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) o[dt][i] *= alpha;
+          o[dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(lf_i16x4, vf),
+                                                            __builtin_bit_cast(lf_i16x4, pb), o[dt], 0, 0, 0);
+        }
+      }
+    }
+    // the other buffer was last read before the barrier of the tile before: it may be written now
+    if (kt + 1 < n_kt) stage(Kl + ((kt + 1) & 1) * LP_KEYS * KSTR);
+    __syncthreads();
+  }
+  if (!row_valid) return;
+  float f = l_run > 0.f ? 1.f / l_run : 0.f;
+  if (gate) f /= 1.f + expf(-(float)gate[(int64_t)my_tok * gate_stride + my_h]);
+  bf16_t* orow = out + ((int64_t)my_tok * heads + my_h) * kv_rank + g * 4;
+#pragma unroll
+  for (int dt = 0; dt < LF_MAXDT; ++dt)
+    if (dt < KDT) {
+      bf16x4 v4;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v4[i] = (bf16_t)(o[dt][i] * f);
+      *(bf16x4*)(orow + dt * 16) = v4;
+    }
+}
+
 // Merges the partial results of `n_splits` (<= 64) workgroups: one wave per (token, head).  Lane s
 // fetches split s's maximum and sum, the weights 2^(m_s - M) are formed once, and the output dims are
 // then summed over the splits with every load independent of the others.  Maxima are in units of
@@ -659,6 +837,33 @@ int tl_latent_flash(const float* qa, const void* latent, const void* rope, const
   if (n_splits > 1)
     hipLaunchKernelGGL(latent_combine_kernel, dim3(n_tokens, heads), dim3(TL_WAVE), 0, stream, part,
                        (const bf16_t*)gate, gate_stride, (bf16_t*)out, n_tokens, heads, kv_rank, n_splits);
+  return tl_launch_status();
+}
+
+// Steps with many query rows: tiles of up to 4 * tpt tokens of one request each (tile lists required).
+int tl_latent_prefill(const float* qa, const void* latent, const void* rope, const int32_t* block_tables,
+                      int max_blocks, const int32_t* tile_req, const int32_t* tile_tok0, const int32_t* tile_ntok,
+                      const int32_t* positions, const void* gate, int64_t gate_stride, void* out, int n_tiles,
+                      int heads, int tpt, int kv_rank, int rot, int block_size, float scale, hipStream_t stream) {
+  if (n_tiles <= 0) return TL_OK;
+  if (heads <= 0 || kv_rank <= 0 || kv_rank % 16 || kv_rank > 16 * LF_MAXDT || rot < 0 || rot % 8 ||
+      kv_rank + rot > 32 * LF_MAXKS || block_size <= 0 || max_blocks <= 0 || !tile_req || !tile_tok0 || !tile_ntok ||
+      tpt != 16 / (heads < 16 ? heads : 16) || (heads + 15) / 16 > 65535)
+    return TL_ERR_ARG;
+  const int WP = (kv_rank + rot + 31) / 32 * 32;
+  // two staged tiles and the four waves' lower query terms: at most 150 KB (the default limit is 64 KB)
+  const size_t lds = (size_t)(2 * LP_KEYS + LF_WAVES * 16) * (WP + LF_PAD) * 2;
+  static int granted_prefill = 0;
+  if ((int)lds > granted_prefill) {
+    if (hipFuncSetAttribute((const void*)latent_prefill_bf16_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)lds) != hipSuccess)
+      return TL_ERR_LAUNCH;
+    granted_prefill = (int)lds;
+  }
+  dim3 g(n_tiles, (heads + 15) / 16), b(LF_WAVES * TL_WAVE);
+  hipLaunchKernelGGL(latent_prefill_bf16_kernel, g, b, lds, stream, qa, (const bf16_t*)latent, (const bf16_t*)rope,
+                     block_tables, max_blocks, tile_req, tile_tok0, tile_ntok, positions, (const bf16_t*)gate,
+                     gate_stride, (bf16_t*)out, heads, tpt, kv_rank, rot, block_size, scale);
   return tl_launch_status();
 }
 

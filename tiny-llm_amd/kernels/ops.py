@@ -1290,6 +1290,47 @@ def latent_flash(qa: torch.Tensor, latent: torch.Tensor, rope: Optional[torch.Te
     return out
 
 
+LATENT_PREFILL_ROWS = 64        # from this many query rows on a step's latent attention shares staged key tiles
+
+
+def latent_prefill(qa: torch.Tensor, latent: torch.Tensor, rope: Optional[torch.Tensor], block_tables: torch.Tensor,
+                   tiles, positions: torch.Tensor, out: torch.Tensor, scale: float,
+                   gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """`latent_flash` for steps with many query rows: tiles = (tile_req, tile_tok0, tile_ntok) with at most
+    4 * (16 // min(heads, 16)) tokens of one request each; the four waves of a workgroup share every staged
+    key tile.  Same operands and result otherwise (no split keys)."""
+    _dev(qa, latent, rope, block_tables, positions, out, gate)
+    _i32(block_tables, positions)
+    T, H, W = qa.shape
+    kv_rank = latent.shape[-1]
+    rot = W - kv_rank
+    if not latent_flash_supported(latent.dtype, kv_rank, rot):
+        _fail(f"latent_prefill takes bfloat16 latents of a multiple of 16 up to 512 and rotated dims of a multiple of 8; got {kv_rank}, {rot}")
+    if not (qa.dtype == torch.float32 and qa.is_contiguous() and latent.dim() == 3 and latent.is_contiguous()
+            and block_tables.dim() == 2 and positions.numel() == T and W % 8 == 0):
+        _fail("latent_prefill: queries are contiguous float32 [T, heads, kv_rank + rot], the cache [blocks, block_size, kv_rank]")
+    if rot and not (rope is not None and rope.dtype == latent.dtype and rope.is_contiguous()
+                    and tuple(rope.shape) == (*latent.shape[:2], rot)):
+        _fail("latent_prefill: the rotated-key cache must be [blocks, block_size, rot] of the cache's type")
+    if not (out.dtype == latent.dtype and out.is_contiguous() and tuple(out.shape) == (T, H, kv_rank)):
+        _fail("latent_prefill: the output is contiguous [T, heads, kv_rank] of the cache's type")
+    if gate is not None and not (gate.dtype == latent.dtype and gate.dim() == 2 and gate.stride(1) == 1
+                                 and tuple(gate.shape) == (T, H)):
+        _fail("latent_prefill: the gate is [T, heads] of the cache's type")
+    treq, ttok, tn = tiles
+    _dev(treq, ttok, tn)
+    _i32(treq, ttok, tn)
+    n_tiles = treq.numel()
+    if not (ttok.numel() == n_tiles and tn.numel() == n_tiles):
+        _fail("latent_prefill: the three tile lists have one length")
+    _check(_lib().tl_latent_prefill(_ptr(qa, 16), _ptr(latent, 16), _ptr(rope, 16), _ptr(block_tables),
+                                    c_int(block_tables.shape[1]), _ptr(treq), _ptr(ttok), _ptr(tn), _ptr(positions),
+                                    _ptr(gate), c_int64(gate.stride(0) if gate is not None else 0), _ptr(out, 8),
+                                    c_int(n_tiles), c_int(H), c_int(16 // min(H, 16)), c_int(kv_rank), c_int(rot),
+                                    c_int(latent.shape[1]), c_float(scale), _stream()), "latent_prefill")
+    return out
+
+
 HEAD_PRODUCT_ROWS = 32      # up to this many rows the per-head products of a step run as ONE launch
 HEAD_PRODUCT_INNER = 1024
 

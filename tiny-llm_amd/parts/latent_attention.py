@@ -155,6 +155,11 @@ class LatentAttention(Mixer):
             # bfloat16: on the matrix cores, 16 heads of a token (or 16 / heads tokens) a tile
             decode = ctx.max_q_len == 1 and T == ctx.num_requests
             tpt = 16 // min(H, 16)
+            if not decode and T >= ops.LATENT_PREFILL_ROWS:
+                # many rows: four times the tokens a workgroup, which share every staged key tile
+                ops.latent_prefill(qa, latent, rope, ctx.block_tables[cache.group], ctx.attention_tiles(4 * tpt),
+                                   ctx.positions, mix, self.scale, gate)
+                return self._project_heads(mix, residual, few, many)
             tiles = None if decode else ctx.attention_tiles(tpt)
             n_tiles = T if decode else tiles[0].numel()
             n_splits = ops.latent_key_splits(n_tiles * -(-H // 16), ctx.max_seq_len)
@@ -166,6 +171,12 @@ class LatentAttention(Mixer):
         else:
             ops.latent_attention(qa, latent, rope, ctx.block_tables[cache.group], ctx.req_of_token, ctx.positions,
                                  mix, self.scale, gate)
+        return self._project_heads(mix, residual, few, many)
+
+    def _project_heads(self, mix, residual, few: bool, many: bool):
+        """W_o concat_n(W_uv,n mix_n), with the per-head products as one launch where a kernel takes them."""
+        T, H, KR = mix.shape
+        V, dev = self.value_dim, mix.device
         o = ops.scratch("latent_heads", (T, H * V), self.dtype, dev)
         if few:
             ops.head_products(mix, self.w_uv_few, o.view(T, H, V))
