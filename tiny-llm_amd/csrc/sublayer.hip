@@ -12,10 +12,10 @@ constexpr int kWaves = kThreads / TL_WAVE;
 
 // x[t] += scale * w * y[t] / sqrt(mean(y[t]^2) + eps); copy[t] = x[t] in TC (optional).
 // One workgroup per row.  `w` is the norm's effective weight, `scale` (optional) a factor per channel.
-// Rows of up to kKeep * kThreads elements stay in registers between the two passes, and what the second
-// pass needs (x, w, scale) is requested before the sum of squares is known.
-constexpr int kKeep = 32;
-template <typename TC>
+// Rows of up to KEEP * kThreads elements stay in registers between the two passes, and what the second
+// pass needs (x, w, scale) is requested before the sum of squares is known (KEEP 8 for rows of up to
+// 2,048 elements, 32 up to 8,192; longer rows are read twice).
+template <typename TC, int KEEP>
 __global__ __launch_bounds__(kThreads) void norm_scale_add_kernel(const float* __restrict__ y,
                                                                   const float* __restrict__ w,
                                                                   const float* __restrict__ scale,
@@ -25,10 +25,10 @@ __global__ __launch_bounds__(kThreads) void norm_scale_add_kernel(const float* _
   const float* src = y + (int64_t)blockIdx.x * hidden;
   float* dst = x + (int64_t)blockIdx.x * hidden;
   float ss = 0.f;
-  if (hidden <= kKeep * kThreads) {
-    float yv[kKeep], xv[kKeep], wv[kKeep];
+  if (hidden <= KEEP * kThreads) {
+    float yv[KEEP], xv[KEEP], wv[KEEP];
 #pragma unroll
-    for (int i = 0; i < kKeep; ++i) {
+    for (int i = 0; i < KEEP; ++i) {
       const int j = threadIdx.x + i * kThreads;
       const bool in = j < hidden;
       yv[i] = in ? src[j] : 0.f;
@@ -39,7 +39,7 @@ __global__ __launch_bounds__(kThreads) void norm_scale_add_kernel(const float* _
     ss = block_sum<kWaves>(ss, red);
     const float r = 1.f / sqrtf(ss / (float)hidden + eps);
 #pragma unroll
-    for (int i = 0; i < kKeep; ++i) {
+    for (int i = 0; i < KEEP; ++i) {
       const int j = threadIdx.x + i * kThreads;
       if (j < hidden) {
         const float s = xv[i] + yv[i] * r * wv[i];
@@ -99,10 +99,15 @@ int tl_norm_scale_add(const float* y, const float* w, const float* scale, float*
   if (n_rows <= 0) return TL_OK;
   if (hidden <= 0) return TL_ERR_ARG;
   dim3 g(n_rows), b(kThreads);
-  if (copy_dtype == 1)
-    hipLaunchKernelGGL(norm_scale_add_kernel<bf16_t>, g, b, 0, stream, y, w, scale, x, (bf16_t*)copy, hidden, eps);
+  const bool few = hidden <= 8 * kThreads;
+  if (copy_dtype == 1 && few)
+    hipLaunchKernelGGL((norm_scale_add_kernel<bf16_t, 8>), g, b, 0, stream, y, w, scale, x, (bf16_t*)copy, hidden, eps);
+  else if (copy_dtype == 1)
+    hipLaunchKernelGGL((norm_scale_add_kernel<bf16_t, 32>), g, b, 0, stream, y, w, scale, x, (bf16_t*)copy, hidden, eps);
+  else if (copy_dtype == 0 && few)
+    hipLaunchKernelGGL((norm_scale_add_kernel<float, 8>), g, b, 0, stream, y, w, scale, x, (float*)copy, hidden, eps);
   else if (copy_dtype == 0)
-    hipLaunchKernelGGL(norm_scale_add_kernel<float>, g, b, 0, stream, y, w, scale, x, (float*)copy, hidden, eps);
+    hipLaunchKernelGGL((norm_scale_add_kernel<float, 32>), g, b, 0, stream, y, w, scale, x, (float*)copy, hidden, eps);
   else
     return TL_ERR_ARG;
   return tl_launch_status();
