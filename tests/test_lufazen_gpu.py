@@ -232,7 +232,8 @@ def test_latent_attention_finds_one_key(dtype):
     splits = 3 if flash and "split" in dtype else 1
     dtype = torch.bfloat16 if flash else dtype
     g = torch.Generator().manual_seed(5)
-    n, kv_rank, rot, block, heads = 700, 48 if flash else 40, 8, 16, 3
+    # the matrix-core kernels with more heads than one tile of 16 rows holds, and not a multiple of it
+    n, kv_rank, rot, block, heads = 700, 48 if flash else 40, 8, 16, 20 if flash else 3
     lat = torch.randn(n, kv_rank, generator=g)
     lat = lat / lat.norm(dim=1, keepdim=True)
     rope = torch.randn(n, rot, generator=g) * 0.1
@@ -244,9 +245,10 @@ def test_latent_attention_finds_one_key(dtype):
     qa = torch.zeros(T, heads, kv_rank + rot)
     for i, (pos, key) in enumerate(cases):
         for h in range(heads):
-            qa[i, h, :kv_rank] = 60.0 * lat[key]
+            # head 0 aims at the case's key, the others at keys of their own around it
+            qa[i, h, :kv_rank] = 60.0 * lat[(key + 7 * h) % (pos + 1)]
             if pos + 1 < n:                       # the key behind the query would win if it were seen
-                qa[i, h, :kv_rank] += 90.0 * lat[pos + 1] * (1.0 if key != pos + 1 else 0.0)
+                qa[i, h, :kv_rank] += 90.0 * lat[pos + 1]
     positions = torch.tensor([c[0] for c in cases], dtype=torch.int32, device="cuda")
     bt = torch.tensor([table + [0] * (64 - len(table))], dtype=torch.int32, device="cuda")
     out = torch.empty(T, heads, kv_rank, dtype=dtype, device="cuda")
@@ -266,13 +268,12 @@ def test_latent_attention_finds_one_key(dtype):
     # the plain softmax over the visible keys
     lat_r, rope_r = lat.to(dtype).double(), rope.to(dtype).double()
     for i, (pos, key) in enumerate(cases):
-        s = qa[i, 0, :kv_rank].double() @ lat_r[:pos + 1].T + qa[i, 0, kv_rank:].double() @ rope_r[:pos + 1].T
-        want = torch.softmax(s, dim=0) @ lat_r[:pos + 1]
-        got = out[i, 0].double().cpu()
-        assert torch.isfinite(got).all()
-        assert (got - want).abs().max() < (2e-5 if dtype == torch.float32 else 1e-2), (pos, key)
-        for h in range(1, heads):
-            assert torch.equal(out[i, h], out[i, 0])
+        for h in range(heads):
+            s = qa[i, h, :kv_rank].double() @ lat_r[:pos + 1].T + qa[i, h, kv_rank:].double() @ rope_r[:pos + 1].T
+            want = torch.softmax(s, dim=0) @ lat_r[:pos + 1]
+            got = out[i, h].double().cpu()
+            assert torch.isfinite(got).all()
+            assert (got - want).abs().max() < (2e-5 if dtype == torch.float32 else 1e-2), (pos, key, h)
 
 
 def test_delta_rule_state_over_slots_and_tiny_portions():
@@ -445,3 +446,40 @@ def test_random_weights_from_a_configuration():
     out = eng.generate([random_tokens(20, cfg["vocab"], 1), random_tokens(3, cfg["vocab"], 2)],
                        SamplingParams.greedy(8, ignore_eos=True))
     assert [len(o) for o in out] == [8, 8] and all(0 <= t < cfg["vocab"] for o in out for t in o)
+
+
+def test_latent_prefill_tiles_of_several_tokens():
+    """The kernel of steps with many rows on tiles that hold several tokens: one request's 13 consecutive
+    tokens in tiles of four (the last one of a single token), 20 heads (two tiles of heads, the second partly
+    used), each head aiming at a key of its own; and 5 heads, where a wave holds three tokens."""
+    from tiny_llm_amd.kernels import ops
+    g = torch.Generator().manual_seed(8)
+    n, kv_rank, rot, block = 420, 64, 16, 8
+    lat = torch.randn(n, kv_rank, generator=g)
+    lat = lat / lat.norm(dim=1, keepdim=True)
+    rope = torch.randn(n, rot, generator=g) * 0.1
+    table = torch.randperm(64, generator=g)[: -(-n // block)].tolist()
+    pages_l, pages_r = _paged(lat, table, block, 64, torch.bfloat16), _paged(rope, table, block, 64, torch.bfloat16)
+    bt = torch.tensor([table + [0] * (64 - len(table))], dtype=torch.int32, device="cuda")
+    lat_r, rope_r = lat.to(torch.bfloat16).double(), rope.to(torch.bfloat16).double()
+    for heads, first in ((20, 300), (5, 27)):
+        T = 13
+        per_tile = 4 * (16 // min(heads, 16))
+        positions = torch.arange(first, first + T, dtype=torch.int32)
+        qa = torch.randn(T, heads, kv_rank + rot, generator=g) * 0.3
+        for t in range(T):
+            for h in range(heads):
+                qa[t, h, :kv_rank] += 50.0 * lat[(11 * h + 3 * t) % (first + t + 1)]
+        starts = list(range(0, T, per_tile))
+        tiles = (torch.zeros(len(starts), dtype=torch.int32, device="cuda"),
+                 torch.tensor(starts, dtype=torch.int32, device="cuda"),
+                 torch.tensor([min(per_tile, T - s0) for s0 in starts], dtype=torch.int32, device="cuda"))
+        gate = torch.randn(T, heads, generator=g).to(torch.bfloat16)
+        out = torch.empty(T, heads, kv_rank, dtype=torch.bfloat16, device="cuda")
+        ops.latent_prefill(qa.cuda(), pages_l, pages_r, bt, tiles, positions.cuda(), out, 0.7, gate.cuda())
+        for t in range(T):
+            p = first + t
+            for h in range(heads):
+                s = (qa[t, h, :kv_rank].double() @ lat_r[:p + 1].T + qa[t, h, kv_rank:].double() @ rope_r[:p + 1].T) * 0.7
+                want = torch.softmax(s, dim=0) @ lat_r[:p + 1] * torch.sigmoid(gate[t, h].double())
+                assert (out[t, h].double().cpu() - want).abs().max() < 1e-2, (heads, t, h)
