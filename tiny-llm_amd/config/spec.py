@@ -35,6 +35,7 @@ class LayerSpec:
     prefix: str                 # weight-name prefix, e.g. "model.layers.3"
     block: str                  # arrangement, e.g. "pre_norm"
     parts: Mapping[str, PartSpec]
+    block_params: Mapping[str, Any] = field(default_factory=dict)     # the arrangement's own constants
 
 
 def pre_norm_layer(prefix: str, mixer_norm: PartSpec, mixer: PartSpec, ffn_norm: PartSpec, ffn: PartSpec,

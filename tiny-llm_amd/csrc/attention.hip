@@ -30,7 +30,7 @@ __global__ __launch_bounds__(TL_WAVE) void paged_attention_kernel(
     const T* __restrict__ v_cache, const int32_t* __restrict__ block_tables, int max_blocks,
     const int32_t* __restrict__ req_of_token, const int32_t* __restrict__ positions,
     T* __restrict__ out, int64_t out_stride, int nq, int nkv, int hd, int block_size, float scale,
-    int window) {
+    int window, int sink) {
   __shared__ float qs[kMaxHd];
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int r = req_of_token[t];
@@ -82,6 +82,8 @@ __global__ __launch_bounds__(TL_WAVE) void paged_attention_kernel(
     }
     m = m_new;
   }
+  // a sink: one more term in the denominator, exp(0 - m) in the scores' own scale, that carries no value
+  if (sink) l += expf(-m);
   T* orow = out + (int64_t)t * out_stride + (int64_t)h * hd;
 #pragma unroll
   for (int i = 0; i < kDPL; ++i) {
@@ -1378,7 +1380,7 @@ extern "C" {
 int tl_paged_attention(const void* q, int64_t q_stride, const void* k_cache, const void* v_cache,
                        const int32_t* block_tables, int max_blocks, const int32_t* req_of_token,
                        const int32_t* positions, void* out, int64_t out_stride, int n_tokens, int nq,
-                       int nkv, int hd, int block_size, float scale, int window, int dtype,
+                       int nkv, int hd, int block_size, float scale, int window, int sink, int dtype,
                        hipStream_t stream) {
   if (n_tokens <= 0) return TL_OK;
   if (nq <= 0 || nkv <= 0 || nq % nkv || hd <= 0 || hd > kMaxHd || block_size <= 0 || max_blocks <= 0 ||
@@ -1388,11 +1390,11 @@ int tl_paged_attention(const void* q, int64_t q_stride, const void* k_cache, con
   if (dtype == 0)
     hipLaunchKernelGGL(paged_attention_kernel<float>, g, b, 0, stream, (const float*)q, q_stride,
                        (const float*)k_cache, (const float*)v_cache, block_tables, max_blocks, req_of_token,
-                       positions, (float*)out, out_stride, nq, nkv, hd, block_size, scale, window);
+                       positions, (float*)out, out_stride, nq, nkv, hd, block_size, scale, window, sink);
   else if (dtype == 1)
     hipLaunchKernelGGL(paged_attention_kernel<bf16_t>, g, b, 0, stream, (const bf16_t*)q, q_stride,
                        (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, max_blocks, req_of_token,
-                       positions, (bf16_t*)out, out_stride, nq, nkv, hd, block_size, scale, window);
+                       positions, (bf16_t*)out, out_stride, nq, nkv, hd, block_size, scale, window, sink);
   else
     return TL_ERR_ARG;
   return tl_launch_status();

@@ -239,21 +239,28 @@ __global__ __launch_bounds__(kRecThreads) void delta_recurrence_kernel(
     if (live && s * DS + i < dim) S_mem[(int64_t)(s * DS + i) * vdim] = S[i];
 }
 
-// z[t, h, :] = w * o[t, h, :] / sqrt(mean(o[t, h, :]^2) + eps) * sigmoid(gate[t, h, :]); one wave per (t, h).
+// z[t, h, :] = scale * w * o[t, h, :] / sqrt(mean(o[t, h, :]^2) + eps) * act(gate[t, h, :]); one wave per (t, h).
+// w is shared by the heads (w_head_stride 0) or each head's own (w_head_stride = vdim); act is the sigmoid
+// (gate_kind 0) or g * sigmoid(g) (gate_kind 1).
 template <typename T>
 __global__ __launch_bounds__(TL_WAVE) void head_norm_gate_kernel(const float* __restrict__ o,
-                                                                 const float* __restrict__ w,
+                                                                 const float* __restrict__ w, int w_head_stride,
                                                                  const float* __restrict__ gate, int64_t gate_stride,
-                                                                 T* __restrict__ z, int heads, int vdim, float eps) {
+                                                                 T* __restrict__ z, int heads, int vdim, float eps,
+                                                                 int gate_kind, float scale) {
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const float* src = o + ((int64_t)t * heads + h) * vdim;
+  const float* wh = w + (int64_t)h * w_head_stride;
   float ss = 0.f;
   for (int j = lane; j < vdim; j += TL_WAVE) ss += src[j] * src[j];
   ss = wave_sum(ss);
-  const float r = 1.f / sqrtf(ss / (float)vdim + eps);
+  const float r = scale / sqrtf(ss / (float)vdim + eps);
   const float* gp = gate + (int64_t)t * gate_stride + (int64_t)h * vdim;
   T* dst = z + ((int64_t)t * heads + h) * vdim;
-  for (int j = lane; j < vdim; j += TL_WAVE) dst[j] = from_f32<T>(src[j] * r * w[j] / (1.f + expf(-gp[j])));
+  for (int j = lane; j < vdim; j += TL_WAVE) {
+    const float g = gp[j], sg = 1.f / (1.f + expf(-g));
+    dst[j] = from_f32<T>(src[j] * r * wh[j] * (gate_kind ? g * sg : sg));
+  }
 }
 
 // Sum over a workgroup of `nw` waves (nw <= 16); `red` is LDS of 16 floats.  Fixed order.
@@ -516,13 +523,16 @@ int tl_delta_decode(const void* p, int64_t p_stride, int conv_off, int b_off, co
   return tl_launch_status();
 }
 
-int tl_head_norm_gate(const float* o, const float* w, const float* gate, int64_t gate_stride, void* z, int n_tokens,
-                      int heads, int vdim, float eps, int dtype, hipStream_t stream) {
+int tl_head_norm_gate(const float* o, const float* w, int w_head_stride, const float* gate, int64_t gate_stride, void* z,
+                      int n_tokens, int heads, int vdim, float eps, int gate_kind, float scale, int dtype,
+                      hipStream_t stream) {
   if (n_tokens <= 0) return TL_OK;
-  if (heads <= 0 || heads > 65535 || vdim <= 0) return TL_ERR_ARG;
+  if (heads <= 0 || heads > 65535 || vdim <= 0 || (w_head_stride != 0 && w_head_stride != vdim) || gate_kind < 0 ||
+      gate_kind > 1)
+    return TL_ERR_ARG;
   dim3 g(n_tokens, heads), b(TL_WAVE);
-  TL_DISPATCH_T(dtype, hipLaunchKernelGGL(head_norm_gate_kernel<T>, g, b, 0, stream, o, w, gate, gate_stride, (T*)z,
-                                          heads, vdim, eps);)
+  TL_DISPATCH_T(dtype, hipLaunchKernelGGL(head_norm_gate_kernel<T>, g, b, 0, stream, o, w, w_head_stride, gate,
+                                          gate_stride, (T*)z, heads, vdim, eps, gate_kind, scale);)
   return tl_launch_status();
 }
 

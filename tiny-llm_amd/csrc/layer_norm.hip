@@ -1,0 +1,113 @@
+// Layer norm with weight and bias, (v - mean) / sqrt(var + eps) * w + b with var the mean squared
+// deviation, in two forms: on the sum of a sublayer's result and the scaled residual stream, written
+// back into the stream (a layer whose norm FOLLOWS the sum: x <- LN(alpha * x + y)), and on gathered
+// rows of the stream for the output head.
+//
+// Statistics, weight, bias and the stream are float32 in both precisions.  The mean is taken first and
+// the variance from the deviations (two sums), not from the mean of squares.
+#include "common.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWaves = kThreads / TL_WAVE;
+
+// v[j] = alpha * x[row, j] + y[row, j] (y optional); x[row] <- LN(v) * w + b (when `inplace`), out[row] likewise
+// in TO (optional).  `rows` (optional) gathers: output row i reads stream row rows[i].  One workgroup a row;
+// rows of up to KEEP * kThreads elements stay in registers between the passes, longer ones are formed again.
+template <typename TO, int KEEP>
+__global__ __launch_bounds__(kThreads) void layer_norm_kernel(const float* __restrict__ y, const float* __restrict__ w,
+                                                              const float* __restrict__ b, float* __restrict__ x,
+                                                              const int32_t* __restrict__ rows, TO* __restrict__ out,
+                                                              int hidden, float alpha, float eps, int inplace) {
+  __shared__ float red[kWaves];
+  const int64_t src_row = rows ? rows[blockIdx.x] : blockIdx.x;
+  float* xr = x + src_row * hidden;
+  const float* yr = y ? y + src_row * hidden : nullptr;
+  TO* dst = out ? out + (int64_t)blockIdx.x * hidden : nullptr;
+  const float inv_n = 1.f / (float)hidden;
+  if (hidden <= KEEP * kThreads) {
+    float v[KEEP];
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < KEEP; ++i) {
+      const int j = threadIdx.x + i * kThreads;
+      v[i] = 0.f;
+      if (j < hidden) v[i] = yr ? fmaf(alpha, xr[j], yr[j]) : alpha * xr[j];
+      s += v[i];
+    }
+    const float mean = block_sum<kWaves>(s, red) * inv_n;
+    float q = 0.f;
+#pragma unroll
+    for (int i = 0; i < KEEP; ++i) {
+      const int j = threadIdx.x + i * kThreads;
+      const float d = j < hidden ? v[i] - mean : 0.f;
+      q += d * d;
+    }
+    const float r = 1.f / sqrtf(block_sum<kWaves>(q, red) * inv_n + eps);
+#pragma unroll
+    for (int i = 0; i < KEEP; ++i) {
+      const int j = threadIdx.x + i * kThreads;
+      if (j < hidden) {
+        const float o = (v[i] - mean) * r * w[j] + b[j];
+        if (inplace) xr[j] = o;
+        if (dst) dst[j] = from_f32<TO>(o);
+      }
+    }
+    return;
+  }
+  float s = 0.f;
+  for (int j = threadIdx.x; j < hidden; j += kThreads) s += yr ? fmaf(alpha, xr[j], yr[j]) : alpha * xr[j];
+  const float mean = block_sum<kWaves>(s, red) * inv_n;
+  float q = 0.f;
+  for (int j = threadIdx.x; j < hidden; j += kThreads) {
+    const float d = (yr ? fmaf(alpha, xr[j], yr[j]) : alpha * xr[j]) - mean;
+    q += d * d;
+  }
+  const float r = 1.f / sqrtf(block_sum<kWaves>(q, red) * inv_n + eps);
+  for (int j = threadIdx.x; j < hidden; j += kThreads) {
+    const float o = ((yr ? fmaf(alpha, xr[j], yr[j]) : alpha * xr[j]) - mean) * r * w[j] + b[j];
+    if (inplace) xr[j] = o;
+    if (dst) dst[j] = from_f32<TO>(o);
+  }
+}
+
+template <typename TO>
+int launch(const float* y, const float* w, const float* b, float* x, const int32_t* rows, TO* out, int n, int hidden,
+           float alpha, float eps, int inplace, hipStream_t stream) {
+  dim3 g(n), blk(kThreads);
+  if (hidden <= 8 * kThreads)
+    hipLaunchKernelGGL((layer_norm_kernel<TO, 8>), g, blk, 0, stream, y, w, b, x, rows, out, hidden, alpha, eps, inplace);
+  else
+    hipLaunchKernelGGL((layer_norm_kernel<TO, 32>), g, blk, 0, stream, y, w, b, x, rows, out, hidden, alpha, eps, inplace);
+  return tl_launch_status();
+}
+
+}  // namespace
+
+extern "C" {
+
+// x[t] <- LN(alpha * x[t] + y[t]) * w + b for n_rows rows (y may be null); copy (optional, copy_dtype 0
+// float32 / 1 bfloat16) receives the new rows too.
+int tl_layer_norm_sum(const float* y, const float* w, const float* b, float* x, void* copy, int n_rows, int hidden,
+                      float alpha, float eps, int copy_dtype, hipStream_t stream) {
+  if (n_rows <= 0) return TL_OK;
+  if (hidden <= 0 || !w || !b || !x) return TL_ERR_ARG;
+  if (copy_dtype == 1) return launch<bf16_t>(y, w, b, x, nullptr, (bf16_t*)copy, n_rows, hidden, alpha, eps, 1, stream);
+  if (copy_dtype == 0) return launch<float>(y, w, b, x, nullptr, (float*)copy, n_rows, hidden, alpha, eps, 1, stream);
+  return TL_ERR_ARG;
+}
+
+// out[i] = LN(x[rows[i] or i]) * w + b; x is not written.
+int tl_layer_norm_rows(const float* x, const int32_t* rows, const float* w, const float* b, void* out, int n,
+                       int hidden, float eps, int out_dtype, hipStream_t stream) {
+  if (n <= 0) return TL_OK;
+  if (hidden <= 0 || !w || !b || !x || !out) return TL_ERR_ARG;
+  if (out_dtype == 1)
+    return launch<bf16_t>(nullptr, w, b, const_cast<float*>(x), rows, (bf16_t*)out, n, hidden, 1.f, eps, 0, stream);
+  if (out_dtype == 0)
+    return launch<float>(nullptr, w, b, const_cast<float*>(x), rows, (float*)out, n, hidden, 1.f, eps, 0, stream);
+  return TL_ERR_ARG;
+}
+
+}  // extern "C"

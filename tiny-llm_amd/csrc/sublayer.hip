@@ -84,6 +84,21 @@ __global__ void clamped_glu_kernel(const T* __restrict__ gate_up, T* __restrict_
   z[i] = from_f32<T>(g / (1.f + expf(-alpha * g)) * (u + shift));
 }
 
+// z[t, j] = gelu(gate_up[t, j]) * gate_up[t, inter + j], gelu in its tanh form:
+// 0.5 g (1 + tanh(sqrt(2 / pi) (g + 0.044715 g^3))).
+template <typename T>
+__global__ void gelu_glu_kernel(const T* __restrict__ gate_up, T* __restrict__ z, int64_t total, int inter,
+                                int64_t in_stride) {
+  const int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (i >= total) return;
+  const int64_t t = i / inter;
+  const int j = (int)(i - t * inter);
+  const float g = to_f32(gate_up[t * in_stride + j]);
+  const float u = to_f32(gate_up[t * in_stride + inter + j]);
+  const float act = 0.5f * g * (1.f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
+  z[i] = from_f32<T>(act * u);
+}
+
 __global__ void softcap_kernel(float* __restrict__ x, int64_t total, float cap) {
   const int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
   if (i < total) x[i] = cap * tanhf(x[i] / cap);
@@ -137,6 +152,21 @@ int tl_clamped_glu(const void* gate_up, void* z, int n_rows, int inter, int64_t 
   else if (dtype == 1)
     hipLaunchKernelGGL(clamped_glu_kernel<bf16_t>, g, b, 0, stream, (const bf16_t*)gate_up, (bf16_t*)z, total, inter,
                        in_stride, limit, alpha, shift);
+  else
+    return TL_ERR_ARG;
+  return tl_launch_status();
+}
+
+int tl_gelu_glu(const void* gate_up, void* z, int n_rows, int inter, int64_t in_stride, int dtype, hipStream_t stream) {
+  if (n_rows <= 0) return TL_OK;
+  if (inter <= 0 || in_stride < 2 * (int64_t)inter) return TL_ERR_ARG;
+  const int64_t total = (int64_t)n_rows * inter;
+  dim3 g((unsigned)ceil_div64(total, kThreads)), b(kThreads);
+  if (dtype == 0)
+    hipLaunchKernelGGL(gelu_glu_kernel<float>, g, b, 0, stream, (const float*)gate_up, (float*)z, total, inter, in_stride);
+  else if (dtype == 1)
+    hipLaunchKernelGGL(gelu_glu_kernel<bf16_t>, g, b, 0, stream, (const bf16_t*)gate_up, (bf16_t*)z, total, inter,
+                       in_stride);
   else
     return TL_ERR_ARG;
   return tl_launch_status();

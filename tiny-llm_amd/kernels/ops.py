@@ -604,9 +604,10 @@ ROPE_PAIRINGS = ("half", "interleaved")     # the rotation kernel's pairings, by
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                     block_tables: torch.Tensor, req_of_token: torch.Tensor, positions: torch.Tensor,
                     out: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, scale: float,
-                    window: int = 0) -> torch.Tensor:
+                    window: int = 0, sink: bool = False) -> torch.Tensor:
     """Causal attention of every row of q (at its absolute position) over its
-    request's cached keys 0..position (the last `window` of them if window > 0)."""
+    request's cached keys 0..position (the last `window` of them if window > 0).
+    sink: the softmax's denominator has one more term, exp(0), that carries no value."""
     _dev(q, k_cache, v_cache, block_tables, req_of_token, positions, out)
     _rows_2d(q, "q")
     _rows_2d(out, "attention output")
@@ -632,7 +633,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         _ptr(q), c_int64(q.stride(0)), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
         c_int(block_tables.shape[1]), _ptr(req_of_token), _ptr(positions), _ptr(out), c_int64(out.stride(0)),
         c_int(T), c_int(num_heads), c_int(num_kv_heads), c_int(head_dim), c_int(k_cache.shape[2]),
-        c_float(scale), c_int(window), c_int(_dt(q)), _stream()), "paged_attention")
+        c_float(scale), c_int(window), c_int(1 if sink else 0), c_int(_dt(q)), _stream()), "paged_attention")
     return out
 
 
@@ -1511,17 +1512,294 @@ def delta_decode(p: torch.Tensor, conv_off: int, b_off: int, low: torch.Tensor, 
 
 
 def head_norm_gate(o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, out: torch.Tensor, heads: int,
-                   vdim: int, eps: float) -> torch.Tensor:
-    """out[t, h, :] = weight * o[t, h, :] / sqrt(mean(o[t, h, :]^2) + eps) * sigmoid(gate[t, h, :]);
-    o float32 [T, heads * vdim], gate float32 [T, heads * vdim] (a view with a row stride is fine)."""
+                   vdim: int, eps: float, gate_kind: str = "sigmoid", scale: float = 1.0) -> torch.Tensor:
+    """out[t, h, :] = scale * weight * o[t, h, :] / sqrt(mean(o[t, h, :]^2) + eps) * act(gate[t, h, :]);
+    o float32 [T, heads * vdim], gate float32 [T, heads * vdim] (a view with a row stride is fine);
+    weight [vdim] (shared by the heads) or [heads * vdim]; act "sigmoid" or "silu" (g * sigmoid(g))."""
     _dev(o, weight, gate, out)
     T = out.shape[0]
     _f32_vec(o, T * heads * vdim, "head_norm_gate input")
-    _f32_vec(weight, vdim, "the head norm's weight")
+    per_head = weight.numel() == heads * vdim and heads > 1
+    _f32_vec(weight, heads * vdim if per_head else vdim, "the head norm's weight")
+    if gate_kind not in ("sigmoid", "silu"):
+        _fail(f"head_norm_gate: unknown gate {gate_kind!r}")
     if not (gate.dtype == torch.float32 and gate.dim() == 2 and gate.stride(1) == 1
             and tuple(gate.shape) == (T, heads * vdim) and out.is_contiguous() and tuple(out.shape) == (T, heads * vdim)):
         _fail("head_norm_gate: gate and output are [T, heads * vdim]")
-    _check(_lib().tl_head_norm_gate(_ptr(o), _ptr(weight), _ptr(gate), c_int64(gate.stride(0)), _ptr(out), c_int(T),
-                                    c_int(heads), c_int(vdim), c_float(eps), c_int(_dt(out)), _stream()),
+    _check(_lib().tl_head_norm_gate(_ptr(o), _ptr(weight), c_int(vdim if per_head else 0), _ptr(gate),
+                                    c_int64(gate.stride(0)), _ptr(out), c_int(T), c_int(heads), c_int(vdim), c_float(eps),
+                                    c_int(1 if gate_kind == "silu" else 0), c_float(scale), c_int(_dt(out)), _stream()),
            "head_norm_gate")
+    return out
+
+
+# ------------------------------------------------- norm after the sum, with weight and bias
+def layer_norm_sum(y: Optional[torch.Tensor], weight: torch.Tensor, bias: torch.Tensor, x: torch.Tensor, alpha: float,
+                   eps: float, copy: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x[t] <- (v - mean(v)) / sqrt(var(v) + eps) * weight + bias with v = alpha * x[t] + y[t] (y None: alpha * x[t]),
+    in place, float32; `copy` ([T, H], any element type of the engine) receives the new rows too."""
+    _dev(y, weight, bias, x, copy)
+    if not (x.dtype == torch.float32 and x.dim() == 2 and x.is_contiguous()):
+        _fail("layer_norm_sum: the stream is contiguous float32 [T, H]")
+    T, H = x.shape
+    if y is not None and not (y.dtype == torch.float32 and y.is_contiguous() and tuple(y.shape) == (T, H)):
+        _fail("layer_norm_sum: the sublayer's result is contiguous float32 [T, H]")
+    _f32_vec(weight, H, "the layer norm's weight")
+    _f32_vec(bias, H, "the layer norm's bias")
+    if copy is not None and not (copy.is_contiguous() and tuple(copy.shape) == (T, H)):
+        _fail("layer_norm_sum: the copy is contiguous [T, H]")
+    _check(_lib().tl_layer_norm_sum(_ptr(y), _ptr(weight), _ptr(bias), _ptr(x), _ptr(copy), c_int(T), c_int(H),
+                                    c_float(alpha), c_float(eps), c_int(_dt(copy) if copy is not None else 0), _stream()),
+           "layer_norm_sum")
+    return x
+
+
+def layer_norm_rows(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps: float, out: torch.Tensor,
+                    rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[i] = layer norm of x[rows[i] or i] (float32 [T, H]) times weight plus bias."""
+    _dev(x, weight, bias, out, rows)
+    if not (x.dtype == torch.float32 and x.dim() == 2 and x.is_contiguous()):
+        _fail("layer_norm_rows: the stream is contiguous float32 [T, H]")
+    H, n = x.shape[1], out.shape[0]
+    _f32_vec(weight, H, "the layer norm's weight")
+    _f32_vec(bias, H, "the layer norm's bias")
+    if not (out.dim() == 2 and out.is_contiguous() and out.shape[1] == H):
+        _fail("layer_norm_rows: the output is contiguous [n, H]")
+    if rows is None:
+        _need(n == x.shape[0], "layer_norm_rows: output rows must match input rows")
+    else:
+        _i32(rows)
+        _need(rows.numel() == n, "layer_norm_rows: one row index per output row")
+    _check(_lib().tl_layer_norm_rows(_ptr(x), _ptr(rows), _ptr(weight), _ptr(bias), _ptr(out), c_int(n), c_int(H),
+                                     c_float(eps), c_int(_dt(out)), _stream()), "layer_norm_rows")
+    return out
+
+
+# ------------------------------------------- queries and keys between their product and the attention
+def qk_prepare(p: torch.Tensor, bias: Optional[torch.Tensor], positions: torch.Tensor, cos: Optional[torch.Tensor],
+               sin: Optional[torch.Tensor], slot_mapping: Optional[torch.Tensor], q_out: torch.Tensor,
+               k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor], num_heads: int, num_kv_heads: int,
+               head_dim: int, rot: int, pairing: str, unit_norm: bool, eps: float, values_are_keys: bool,
+               v_off: int = -1) -> torch.Tensor:
+    """From the float32 product p [T, >= (heads + kv_heads) * head_dim] (query heads, then key heads): bias added,
+    the first `rot` dims of every head rotated by the token's position, every head divided by its root mean square
+    (unit_norm); queries go to q_out [T, heads * head_dim], keys into k_cache at the tokens' slots.  values_are_keys:
+    the keys as projected (bias added, before rotation and norm) go into v_cache; else the value heads at column
+    v_off of p do (v_off < 0: no values are written).  A negative slot stores nothing."""
+    _dev(p, bias, positions, cos, sin, slot_mapping, q_out, k_cache, v_cache)
+    _rows_2d(p, "qk_prepare input")
+    _rows_2d(q_out, "qk_prepare queries")
+    T = p.shape[0]
+    width = (num_heads + num_kv_heads) * head_dim
+    _need(p.dtype == torch.float32 and p.shape[1] >= width, f"qk_prepare: the product is float32 [T, >= {width}]")
+    _need(tuple(q_out.shape) == (T, num_heads * head_dim), "qk_prepare: queries are [T, heads * head_dim]")
+    _need(head_dim % 2 == 0 and 0 < head_dim <= MAX_HEAD_DIM and 0 <= rot <= head_dim and rot % 2 == 0,
+          f"qk_prepare: head_dim {head_dim} must be even and at most {MAX_HEAD_DIM}, rot even and within it")
+    if pairing not in ROPE_PAIRINGS:
+        _fail(f"rotary pairing {pairing!r} is not built; known: {', '.join(ROPE_PAIRINGS)}")
+    if bias is not None:
+        _f32_vec(bias, width, "qk_prepare bias")
+    _i32(positions)
+    _need(positions.numel() == T, "qk_prepare: one position per token")
+    if rot:
+        for t in (cos, sin):
+            _need(t is not None and t.dtype == torch.float32 and t.is_contiguous() and t.dim() == 2
+                  and t.shape[1] == rot // 2, "qk_prepare: angle tables are float32 [positions, rot / 2]")
+    block = 1
+    if slot_mapping is not None:
+        _i32(slot_mapping)
+        _need(slot_mapping.numel() == T, "qk_prepare: one slot per token")
+        for c in (k_cache, v_cache):
+            _need(c is not None and c.is_contiguous() and c.dim() == 4 and c.shape[1] == num_kv_heads
+                  and c.shape[3] == head_dim and c.dtype == q_out.dtype,
+                  "qk_prepare: caches are contiguous [blocks, kv_heads, block, head_dim] of the queries' type")
+        _need(k_cache.shape == v_cache.shape, "qk_prepare: key and value caches have one shape")
+        block = k_cache.shape[2]
+    if not values_are_keys and v_off >= 0:
+        _need(p.shape[1] >= v_off + num_kv_heads * head_dim, "qk_prepare: the value heads lie within the product's rows")
+    _check(_lib().tl_qk_prepare(_ptr(p), c_int64(p.stride(0)), _ptr(bias), _ptr(positions), _ptr(cos), _ptr(sin),
+                                _ptr(slot_mapping), _ptr(q_out), c_int64(q_out.stride(0)), _ptr(k_cache), _ptr(v_cache),
+                                c_int(T), c_int(num_heads), c_int(num_kv_heads), c_int(head_dim), c_int(rot),
+                                c_int(ROPE_PAIRINGS.index(pairing)), c_int(1 if unit_norm else 0), c_float(eps),
+                                c_int(1 if values_are_keys else 0), c_int(v_off), c_int(block), c_int(_dt(q_out)),
+                                _stream()), "qk_prepare")
+    return q_out
+
+
+def head_gate(a: torch.Tensor, g: torch.Tensor, out: torch.Tensor, heads: int, head_dim: int, scale: float = 1.0):
+    """out[t, h, :] = a[t, h, :] * sigmoid(g[t, h]) * scale; a and out [T, heads * head_dim] of one type (out may be a),
+    g float32 [T, heads] (a view with a row stride is fine)."""
+    _dev(a, g, out)
+    _rows_2d(a, "head_gate input")
+    _rows_2d(out, "head_gate output")
+    _rows_2d(g, "head_gate gates")
+    T = a.shape[0]
+    _need(tuple(a.shape) == (T, heads * head_dim) and a.shape == out.shape and a.dtype == out.dtype,
+          "head_gate: input and output are [T, heads * head_dim] of one type")
+    _need(g.dtype == torch.float32 and tuple(g.shape) == (T, heads), "head_gate: gates are float32 [T, heads]")
+    _check(_lib().tl_head_gate(_ptr(a), c_int64(a.stride(0)), _ptr(g), c_int64(g.stride(0)), _ptr(out),
+                               c_int64(out.stride(0)), c_int(T), c_int(heads), c_int(head_dim), c_float(scale),
+                               c_int(_dt(a)), _stream()), "head_gate")
+    return out
+
+
+def gelu_glu(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[t, j] = gelu_tanh(gate_up[t, j]) * gate_up[t, F + j]; gate_up [T, 2F], out [T, F] contiguous, one type."""
+    _dev(gate_up, out)
+    _rows_2d(gate_up, "gelu_glu input")
+    T, F = out.shape
+    _need(gate_up.shape[0] == T and gate_up.shape[1] == 2 * F and out.is_contiguous() and out.dtype == gate_up.dtype,
+          "gelu_glu: input [T, 2F], output contiguous [T, F] of the same type")
+    _check(_lib().tl_gelu_glu(_ptr(gate_up), _ptr(out), c_int(T), c_int(F), c_int64(gate_up.stride(0)),
+                              c_int(_dt(out)), _stream()), "gelu_glu")
+    return out
+
+
+# -------------------------------------------------------- time mixing with a decaying state
+TIME_MIX_MAX_DIM = 256      # key channels of a head (csrc/time_mix.hip)
+TIME_MIX_SLICE = 16
+
+
+def time_mix_slices(dim: int) -> int:
+    """Slices of 16 key channels a head's state is cut into (a power of two)."""
+    p = 1
+    while p * TIME_MIX_SLICE < dim:
+        p *= 2
+    return p
+
+
+def time_mix_state_floats(heads: int, dim: int, vdim: int) -> int:
+    """Floats of a request's state row that hold S, in the recurrence kernel's own layout."""
+    return heads * TIME_MIX_SLICE * time_mix_slices(dim) * vdim
+
+
+def shift_mix(h: torch.Tensor, state: torch.Tensor, prev_off: int, req_of_token: torch.Tensor, cu_seqlens: torch.Tensor,
+              state_slots: torch.Tensor, mu: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[m, t] = h[t] + (h[t - 1] - h[t]) * mu[m]; for the first token a request brings in this step h[t - 1] is what
+    its state row keeps at prev_off.  h [T, W] and out [M, T, W] of one type, mu float32 [M, W], state float32 rows."""
+    _dev(h, state, req_of_token, cu_seqlens, state_slots, mu, out)
+    _rows_2d(h, "shift_mix input")
+    T, W = h.shape
+    M = mu.shape[0]
+    _need(mu.dtype == torch.float32 and mu.is_contiguous() and tuple(mu.shape) == (M, W), "shift_mix: mu is float32 [M, W]")
+    _need(out.is_contiguous() and tuple(out.shape) == (M, T, W) and out.dtype == h.dtype,
+          "shift_mix: the output is contiguous [M, T, W] of the input's type")
+    _need(state.dtype == torch.float32 and state.dim() == 2 and state.stride(1) == 1 and state.shape[1] >= prev_off + W,
+          "shift_mix: state rows are float32 and hold W values from prev_off")
+    _i32(req_of_token, cu_seqlens, state_slots)
+    _need(req_of_token.numel() == T, "shift_mix: one request index per token")
+    _check(_lib().tl_shift_mix(_ptr(h), c_int64(h.stride(0)), _ptr(state), c_int64(state.stride(0)), c_int64(prev_off),
+                               _ptr(req_of_token), _ptr(cu_seqlens), _ptr(state_slots), _ptr(mu), _ptr(out), c_int(T),
+                               c_int(M), c_int(W), c_int(_dt(h)), _stream()), "shift_mix")
+    return out
+
+
+def shift_save(h: torch.Tensor, state: torch.Tensor, prev_off: int, cu_seqlens: torch.Tensor,
+               state_slots: torch.Tensor) -> None:
+    """The last token every request brings in this step becomes its state row's saved h (float32)."""
+    _dev(h, state, cu_seqlens, state_slots)
+    _rows_2d(h, "shift_save input")
+    W = h.shape[1]
+    R = state_slots.numel()
+    _need(state.dtype == torch.float32 and state.dim() == 2 and state.stride(1) == 1 and state.shape[1] >= prev_off + W,
+          "shift_save: state rows are float32 and hold W values from prev_off")
+    _i32(cu_seqlens, state_slots)
+    _need(cu_seqlens.numel() == R + 1, "shift_save: cu_seqlens has one entry more than there are requests")
+    _check(_lib().tl_shift_save(_ptr(h), c_int64(h.stride(0)), _ptr(state), c_int64(state.stride(0)), c_int64(prev_off),
+                                _ptr(cu_seqlens), _ptr(state_slots), c_int(R), c_int(W), c_int(_dt(h)), _stream()),
+           "shift_save")
+
+
+def time_mix_recurrence(x: torch.Tensor, r_off: int, k_off: int, v_off: int, w_off: int, w0: torch.Tensor,
+                        u: torch.Tensor, state: torch.Tensor, cu_seqlens: torch.Tensor, state_slots: torch.Tensor,
+                        o: torch.Tensor, heads: int, dim: int, vdim: int) -> torch.Tensor:
+    """Per request and head, over the request's tokens of this step in order, S from its state row:
+    o_t = (S + diag(u) k_t v_t^T)^T r_t, then S <- diag(exp(-exp(x_w + w0))) S + k_t v_t^T.
+    x float32 rows with r, k, the decay's pre-activation (heads * dim columns each) and v (heads * vdim) at the
+    given column offsets; o float32 [T, heads * vdim].  A request that brings no token keeps its state."""
+    _dev(x, w0, u, state, cu_seqlens, state_slots, o)
+    _rows_2d(x, "time_mix_recurrence input")
+    T = x.shape[0]
+    R = state_slots.numel()
+    _need(x.dtype == torch.float32, "time_mix_recurrence: the input is float32")
+    _need(0 < dim <= TIME_MIX_MAX_DIM and vdim > 0 and 0 < heads <= 65535 and R <= 65535,
+          f"time_mix_recurrence: heads of 1 to {TIME_MIX_MAX_DIM} key channels")
+    for off, n in ((r_off, heads * dim), (k_off, heads * dim), (w_off, heads * dim), (v_off, heads * vdim)):
+        _need(0 <= off and off + n <= x.shape[1], "time_mix_recurrence: a column range lies outside the input's rows")
+    _f32_vec(w0, heads * dim, "the decay's bias")
+    _f32_vec(u, heads * dim, "the bonus")
+    _f32_vec(o, T * heads * vdim, "time_mix_recurrence output")
+    _need(state.dtype == torch.float32 and state.dim() == 2 and state.stride(1) == 1
+          and state.shape[1] >= time_mix_state_floats(heads, dim, vdim), "time_mix_recurrence: state rows are too short")
+    _i32(cu_seqlens, state_slots)
+    _need(cu_seqlens.numel() == R + 1, "time_mix_recurrence: cu_seqlens has one entry more than there are requests")
+    _check(_lib().tl_time_mix_recurrence(_ptr(x), c_int64(x.stride(0)), c_int(r_off), c_int(k_off), c_int(v_off),
+                                         c_int(w_off), _ptr(w0), _ptr(u), _ptr(state), c_int64(state.stride(0)),
+                                         _ptr(cu_seqlens), _ptr(state_slots), _ptr(o), c_int(R), c_int(heads), c_int(dim),
+                                         c_int(vdim), _stream()), "time_mix_recurrence")
+    return o
+
+
+def tanh_rows(x: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out = tanh(x); x float32 [T, n] (a row stride is fine), out contiguous [T, n] of the engine's type."""
+    _dev(x, out)
+    _rows_2d(x, "tanh input")
+    _need(x.dtype == torch.float32 and out.is_contiguous() and out.shape == x.shape, "tanh: float32 in, contiguous out")
+    _check(_lib().tl_tanh_rows(_ptr(x), c_int64(x.stride(0)), _ptr(out), c_int(x.shape[0]), c_int(x.shape[1]),
+                               c_int(_dt(out)), _stream()), "tanh_rows")
+    return out
+
+
+# ------------------------------------------------------------ experts looked up in a table
+def table_moe_up(a: torch.Tensor, w: torch.Tensor, tokens: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[t * top + j] = w[table[tokens[t], j]] @ a[t]; a [T, K], w [E, N, K] of one type, table int32 [vocab, top],
+    out contiguous [T * top, N]."""
+    _dev(a, w, tokens, table, out)
+    _rows_2d(a, "table_moe_up input")
+    T, K = a.shape
+    E, N, _ = w.shape
+    V, top = table.shape
+    _need(w.is_contiguous() and w.shape[2] == K and w.dtype == a.dtype == out.dtype, "table_moe_up: w is contiguous [E, N, K]")
+    _need(out.is_contiguous() and tuple(out.shape) == (T * top, N), "table_moe_up: the output is contiguous [T * top, N]")
+    _i32(tokens, table)
+    _need(tokens.numel() == T, "table_moe_up: one token id per row")
+    _check(_lib().tl_table_moe_up(_ptr(a), c_int64(a.stride(0)), _ptr(w), _ptr(tokens), _ptr(table), _ptr(out), c_int(T),
+                                  c_int(top), c_int(E), c_int(V), c_int(N), c_int(K), c_int(_dt(a)), _stream()),
+           "table_moe_up")
+    return out
+
+
+def table_moe_down(z: torch.Tensor, w: torch.Tensor, tokens: torch.Tensor, table: torch.Tensor, out: torch.Tensor,
+                   coef: float, base: Optional[torch.Tensor] = None, base_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[t] = base[t] * base_scale[t] + coef * sum_j w[table[tokens[t], j]] @ z[t * top + j]; z [T * top, K],
+    w [E, N, K], out float32 [T, N] (may be base); base float32 [T, N], base_scale float32 [T], both optional."""
+    _dev(z, w, tokens, table, out, base, base_scale)
+    E, N, K = w.shape
+    V, top = table.shape
+    T = tokens.numel()
+    _need(w.is_contiguous() and z.is_contiguous() and tuple(z.shape) == (T * top, K) and z.dtype == w.dtype,
+          "table_moe_down: z is contiguous [T * top, K], w contiguous [E, N, K]")
+    _need(out.dtype == torch.float32 and out.is_contiguous() and tuple(out.shape) == (T, N),
+          "table_moe_down: the output is contiguous float32 [T, N]")
+    if base is not None:
+        _need(base.dtype == torch.float32 and base.is_contiguous() and base.shape == out.shape,
+              "table_moe_down: base is contiguous float32 [T, N]")
+    if base_scale is not None:
+        _f32_vec(base_scale, T, "table_moe_down base_scale")
+    _i32(tokens, table)
+    _check(_lib().tl_table_moe_down(_ptr(z), _ptr(w), _ptr(tokens), _ptr(table), _ptr(base), _ptr(base_scale), _ptr(out),
+                                    c_int(T), c_int(top), c_int(E), c_int(V), c_int(N), c_int(K), c_float(coef),
+                                    c_int(_dt(z)), _stream()), "table_moe_down")
+    return out
+
+
+def row_dot_sigmoid(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[t] = sigmoid(a[t] . w); a [T, K] and w [K] of one type, out float32 [T]."""
+    _dev(a, w, out)
+    _rows_2d(a, "row_dot_sigmoid input")
+    T, K = a.shape
+    _need(w.is_contiguous() and w.numel() == K and w.dtype == a.dtype, "row_dot_sigmoid: w is [K] of the input's type")
+    _f32_vec(out, T, "row_dot_sigmoid output")
+    _check(_lib().tl_row_dot_sigmoid(_ptr(a), c_int64(a.stride(0)), _ptr(w), _ptr(out), c_int(T), c_int(K),
+                                     c_int(_dt(a)), _stream()), "row_dot_sigmoid")
     return out

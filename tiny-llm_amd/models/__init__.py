@@ -1,2 +1,2 @@
-from . import llama, lufazen  # noqa: F401  (register LlamaForCausalLM, Lufazen)
+from . import llama, lufazen, fofapel  # noqa: F401  (register LlamaForCausalLM, Lufazen, Fofapel)
 from .decoder import Decoder

@@ -44,7 +44,7 @@ class Layer:
                 raise ValueError(f"layer {spec.prefix}: arrangement {spec.block!r} needs a part for role {role!r}")
             ps = spec.parts[role]
             self.by_role[role] = build_part(category, ps, f"{spec.prefix}.{ps.name or role}", dtype, device)
-        self.block = arrangement(self.by_role)
+        self.block = arrangement(self.by_role, **dict(spec.block_params))
 
     def parts(self) -> List[Part]:
         return list(self.by_role.values())

@@ -3,4 +3,4 @@ from .base import (Part, Embedding, Head, Norm, Mixer, FeedForward, PositionEnco
                    NORMS, MIXERS, FEED_FORWARDS, POSITION_ENCODINGS, SCALES, BLOCKS, REGISTRIES, register_embedding,
                    register_head, register_norm, register_mixer, register_feed_forward,
                    register_position_encoding, register_scale, register_block)
-from . import norm, rotary, attention, latent_attention, delta_rule, mlp, block, embedding  # noqa: F401  (fills the registries)
+from . import norm, rotary, attention, latent_attention, delta_rule, time_mix, parallel, mlp, moe, block, embedding  # noqa: F401  (fills the registries)

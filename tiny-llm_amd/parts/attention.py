@@ -84,7 +84,6 @@ class Attention(Mixer):
         attn = ops.scratch("attention_out", (T, self.q_size), self.dtype, residual.device)
         q = qkv[:, :self.q_size]
         flash = ops.flash_attention_supported(self.dtype, self.num_heads, self.num_kv_heads, self.head_dim)
-        group = self.num_heads // self.num_kv_heads
         # decode steps: rotation and cache write ride in the attention kernel
         fuse = flash and ctx.max_q_len == 1 and cache.write and rot == self.head_dim and pairing == "half"
         if not fuse:
@@ -92,6 +91,21 @@ class Attention(Mixer):
             ops.rope_store(qkv, ctx.positions, cos, sin, slots, cache.k if cache.write else None,
                            cache.v if cache.write else None, self.num_heads, self.num_kv_heads, self.head_dim, rot,
                            pairing)
+        self._attend(q, ctx, cache, attn, fused_rope=(cos, sin) if fuse else None)
+        out, prepared = project_into_residual(attn, self.w_o, residual, next_norm)
+        return out if next_norm is None else (out, prepared)
+
+    def _attend(self, q, ctx, cache: LayerCache, attn, fused_rope=None, sink: bool = False):
+        """attn <- attention of the step's query rows q [T, heads * head_dim] over the cache, by the kernel that
+        takes this step's shape.  sink: one more term exp(0) in every softmax's denominator."""
+        T, device = q.shape[0], q.device
+        group = self.num_heads // self.num_kv_heads
+        flash = ops.flash_attention_supported(self.dtype, self.num_heads, self.num_kv_heads, self.head_dim)
+        if sink:
+            # the kernel that takes every size is the one that knows the sink
+            return ops.paged_attention(q, cache.k, cache.v, ctx.block_tables[cache.group], ctx.req_of_token,
+                                       ctx.positions, attn, self.num_heads, self.num_kv_heads, self.head_dim,
+                                       self.scale, self.window, sink=True)
         if flash and ctx.max_q_len > 1:
             # prompt portions: many query rows share each staged key tile
             waves = ops.prefill_tile_waves(T, self.num_heads, self.num_kv_heads)
@@ -101,7 +115,7 @@ class Attention(Mixer):
             scratch = None
             if n_splits > 1:
                 scratch = ops.scratch("attention_partials", (n_splits * T * self.num_heads * (self.head_dim + 2),),
-                                      torch.float32, residual.device)
+                                      torch.float32, device)
             ops.flash_prefill(q, cache.k, cache.v, ctx.block_tables[cache.group], tiles, ctx.positions, attn,
                               self.num_heads, self.num_kv_heads, self.head_dim, self.scale, self.window, waves,
                               n_splits, scratch)
@@ -110,10 +124,10 @@ class Attention(Mixer):
             # workgroups when the context is long)
             # (no tile arrays when every request brings exactly one token: row i is request i)
             tiles = None if T == ctx.num_requests else ctx.attention_tiles(16 // group)
-            n_splits, scratch = self._splits(ctx, T, residual.device)
+            n_splits, scratch = self._splits(ctx, T, device)
             ops.flash_attention(q, cache.k, cache.v, ctx.block_tables[cache.group], tiles, ctx.positions, attn,
                                 self.num_heads, self.num_kv_heads, self.head_dim, self.scale, self.window,
-                                n_splits, scratch, fused_rope=(cos, sin) if fuse else None)
+                                n_splits, scratch, fused_rope=fused_rope)
         elif ops.attention_f32_supported(self.dtype, self.num_heads, self.num_kv_heads, self.head_dim) \
                 and q.stride(0) % 4 == 0:
             # true float32 on the matrix cores; one fixed merge tree, so the same bits whatever the batch
@@ -123,7 +137,7 @@ class Attention(Mixer):
             scratch = None
             if n_chunks > 1:
                 scratch = ops.scratch("attention_partials", (n_chunks * T * self.num_heads * (self.head_dim + 2),),
-                                      torch.float32, residual.device)
+                                      torch.float32, device)
             ops.attention_f32(q, cache.k, cache.v, ctx.block_tables[cache.group], tiles, ctx.positions, attn,
                               self.num_heads, self.num_kv_heads, self.head_dim, self.scale, self.window, n_chunks,
                               scratch)
@@ -131,8 +145,7 @@ class Attention(Mixer):
             ops.paged_attention(q, cache.k, cache.v, ctx.block_tables[cache.group], ctx.req_of_token,
                                 ctx.positions, attn, self.num_heads, self.num_kv_heads, self.head_dim,
                                 self.scale, self.window)
-        out, prepared = project_into_residual(attn, self.w_o, residual, next_norm)
-        return out if next_norm is None else (out, prepared)
+        return attn
 
     def _splits(self, ctx, T: int, device):
         """How many workgroups share one query tile's keys (`ops.decode_key_splits`), and the scratch
@@ -144,4 +157,104 @@ class Attention(Mixer):
                                      torch.float32, device)
 
 
+class NormedAttention(Attention):
+    """Grouped-query attention over the paged cache whose queries and keys are prepared in float32 between
+    their product and the attention kernel, each step an option of its own:
+
+        q, k = W_q h (+ b_q), W_k h (+ b_k)             `bias`
+        v    = k as projected (`values="keys"`, no W_v), or W_v h (`values="projected"`)
+        q, k rotated on the first rotary_dim dims of every head (`position`, either pairing)
+        q, k divided by their root mean square over the head (`qk_norm="unit"`, no weight, `eps`)
+        p_j  = exp(s_j) / (1 + sum exp(s_j))            `sink`: a term of score 0 that carries no value
+        head n's output times sigmoid(W_g h)_n          `head_gate`: one number per token and head
+        result = out_scale * W_o concat_heads(...)
+
+    `window` and `scale` as in `Attention`.  `names`: the tensors' names below the prefix (q, k, v, g, o;
+    a bias is its matrix's name plus `bias_suffix`).  One product reads h for [q | k | (v) | g] and leaves
+    float32; the gate and `out_scale` are applied to the attention's result in float32 before it is
+    rounded for the output product.  With `residual=None` the result is returned by itself in float32."""
+    graph_safe = True
+    accepts_lazy_norm = False
+    prepares_next_norm = False
+
+    def __init__(self, prefix, dtype, device, *, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
+                 position: dict = None, window: int = 0, scale: float = None, bias: bool = False,
+                 values: str = "projected", qk_norm: str = None, eps: float = 1e-6, sink: bool = False,
+                 head_gate: bool = False, out_scale: float = 1.0, names: Dict[str, str] = None,
+                 bias_suffix: str = ".bias", max_position: int = 0):
+        super().__init__(prefix, dtype, device, hidden_size=hidden_size, num_heads=num_heads,
+                         num_kv_heads=num_kv_heads, head_dim=head_dim, position=position, window=window, scale=scale)
+        if values not in ("projected", "keys"):
+            raise ValueError(f"{prefix}: values are 'projected' or 'keys', got {values!r}")
+        if qk_norm not in (None, "unit"):
+            raise ValueError(f"{prefix}: qk_norm is None or 'unit', got {qk_norm!r}")
+        if self.head_dim % 2:
+            raise ValueError(f"{prefix}: head_dim {self.head_dim} must be even")
+        if float(out_scale) != 1.0 and not head_gate:
+            raise ValueError(f"{prefix}: out_scale rides in the head gate's kernel; without a gate it must be 1")
+        self.bias, self.values_are_keys, self.unit_norm = bool(bias), values == "keys", qk_norm == "unit"
+        self.eps, self.sink, self.head_gate, self.out_scale = float(eps), bool(sink), bool(head_gate), float(out_scale)
+        n = {k: k for k in ("q", "k", "v", "g", "o")}
+        n.update(names or {})
+        self.names = {k: f"{prefix}.{v}" for k, v in n.items()}
+        self.bias_suffix = bias_suffix
+        # columns of the product that reads h: q heads, k heads, (v heads,) then the gates at a multiple of 8
+        self.v_off = self.q_size + self.kv_size if not self.values_are_keys else -1
+        used = self.q_size + self.kv_size * (1 if self.values_are_keys else 2)
+        self.g_off = -(-used // 8) * 8
+        self.in_width = self.g_off + (-(-self.num_heads // 8) * 8 if self.head_gate else 0)
+        self.w_in = self.b_in = None
+
+    def weights(self) -> List[WeightSpec]:
+        n, H = self.names, self.hidden_size
+        out = [WeightSpec(n["q"], (self.q_size, H)), WeightSpec(n["k"], (self.kv_size, H))]
+        if self.bias:
+            out += [WeightSpec(n["q"] + self.bias_suffix, (self.q_size,), role="vector", init="zeros"),
+                    WeightSpec(n["k"] + self.bias_suffix, (self.kv_size,), role="vector", init="zeros")]
+        if not self.values_are_keys:
+            out.append(WeightSpec(n["v"], (self.kv_size, H)))
+        if self.head_gate:
+            out.append(WeightSpec(n["g"], (self.num_heads, H)))
+        out.append(WeightSpec(n["o"], (H, self.q_size)))
+        return out
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        n = self.names
+        dev = tensors[n["q"]].device
+        w = torch.zeros((self.in_width, self.hidden_size), dtype=self.dtype, device=dev)
+        w[:self.q_size] = tensors[n["q"]]
+        w[self.q_size:self.q_size + self.kv_size] = tensors[n["k"]]
+        if not self.values_are_keys:
+            w[self.v_off:self.v_off + self.kv_size] = tensors[n["v"]]
+        if self.head_gate:
+            w[self.g_off:self.g_off + self.num_heads] = tensors[n["g"]]
+        self.w_in = w
+        if self.bias:
+            self.b_in = torch.cat([tensors[n["q"] + self.bias_suffix].to(torch.float32),
+                                   tensors[n["k"] + self.bias_suffix].to(torch.float32)]).contiguous()
+        self.w_o = tensors[n["o"]].contiguous()
+
+    def forward(self, h, ctx, cache: LayerCache, state, residual):
+        T, dev = h.shape[0], h.device
+        p = ops.scratch("qk_product", (T, self.in_width), torch.float32, dev)
+        ops.linear(h, self.w_in, p)
+        tables = self.position.rotary_tables()
+        cos, sin, rot = tables if tables is not None else (None, None, 0)
+        pairing = getattr(self.position, "pairing", "half")
+        q = ops.scratch("q_prepared", (T, self.q_size), self.dtype, dev)
+        write = cache.write
+        ops.qk_prepare(p, self.b_in, ctx.positions, cos, sin, ctx.slot_mappings[cache.group] if write else None, q,
+                       cache.k if write else None, cache.v if write else None, self.num_heads, self.num_kv_heads,
+                       self.head_dim, rot, pairing, self.unit_norm, self.eps, self.values_are_keys, self.v_off)
+        attn = ops.scratch("attention_out", (T, self.q_size), self.dtype, dev)
+        self._attend(q, ctx, cache, attn, sink=self.sink)
+        if self.head_gate:
+            ops.head_gate(attn, p[:, self.g_off:self.g_off + self.num_heads], attn, self.num_heads, self.head_dim,
+                          self.out_scale)
+        if residual is None:
+            return ops.linear(attn, self.w_o, ops.scratch("sublayer_out", (T, self.hidden_size), torch.float32, dev))
+        return ops.linear(attn, self.w_o, residual, residual)
+
+
 register_mixer("attention", Attention)
+register_mixer("normed_attention", NormedAttention)

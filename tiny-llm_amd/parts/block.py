@@ -1,13 +1,19 @@
 """Block arrangements.  "pre_norm" is Llama's: x + mixer(norm(x)), then
 x + ffn(norm(x)) (tiny_llm/parser/llama_parser.cpp:194-255).  "output_norm" puts the norm on each
 sublayer's result instead: x + scale * norm(mixer(x)), then x + scale * norm(ffn(x)); the
-sublayers read the residual stream itself."""
+sublayers read the residual stream itself.  "sum_norm" puts the norm behind the sum:
+x <- norm(alpha * x + mixer(x)), then x <- norm(alpha * x + ffn(x)), alpha a constant of the model."""
 from __future__ import annotations
 
 import torch
 
 from ..kernels import ops
 from .base import Block, register_block
+
+
+class StreamCopyWanted:
+    """What an arrangement whose sublayers read the stream itself shows as its `first_norm`: the block
+    in front may hand over the copy of x in the engine's element type instead of a prepared norm."""
 
 
 class PreNormBlock(Block):
@@ -61,9 +67,7 @@ class OutputNormBlock(Block):
              "ffn": "feed_forward", "ffn_norm": "norm", "ffn_scale": "scale"}
     optional = ("mixer_scale", "ffn", "ffn_norm", "ffn_scale")
 
-    class _WantsCopy:
-        """What this arrangement shows as its `first_norm`: the block in front may hand over the
-        copy of x in the engine's element type instead of a prepared norm."""
+    _WantsCopy = StreamCopyWanted
 
     def __init__(self, parts):
         super().__init__(parts)
@@ -104,5 +108,55 @@ class OutputNormBlock(Block):
         return x, copy
 
 
+class SumNormBlock(Block):
+    """x <- norm1(alpha * x + mixer(x)); x <- norm2(alpha * x + ffn(x)).  The sublayers read x itself, are
+    called with `residual=None` and return their result by itself in float32; scaling, sum and norm in
+    float32 are one kernel, which also writes the copy of x in the engine's element type that the next
+    sublayer's products read (in float32 they read x itself).  A layer may have no feed-forward; if it
+    still has a second norm, that norm runs on alpha * x."""
+    roles = {"mixer": "mixer", "mixer_norm": "norm", "ffn": "feed_forward", "ffn_norm": "norm"}
+    optional = ("ffn", "ffn_norm")
+
+    _WantsCopy = StreamCopyWanted
+
+    def __init__(self, parts, alpha: float = 1.0):
+        super().__init__(parts)
+        self.alpha = float(alpha)
+        self.mixer, self.mixer_norm = parts["mixer"], parts["mixer_norm"]
+        self.ffn, self.ffn_norm = parts.get("ffn"), parts.get("ffn_norm")
+        if self.ffn is not None and self.ffn_norm is None:
+            raise ValueError("sum_norm: a feed-forward comes with its norm")
+        for n in (self.mixer_norm, self.ffn_norm):
+            if n is not None and not hasattr(n, "sum_normed"):
+                raise ValueError(f"sum_norm: the norm {type(n).__name__} cannot follow a sum (no sum_normed)")
+        self.first_norm = self._WantsCopy()
+
+    def forward(self, x, ctx, caches, states):
+        return self.forward_chained(x, ctx, caches, states)[0]
+
+    def _copy(self, x):
+        return ops.scratch("stream_copy", x.shape, self.mixer.dtype, x.device, rotate=2)
+
+    def forward_chained(self, x, ctx, caches, states, prepared=None, next_norm=None):
+        """`prepared`: the copy of x in the engine's element type, if the block in front hands one over;
+        returned likewise for the block behind (when `next_norm` says it takes one)."""
+        low = x.dtype != self.mixer.dtype          # the products read a copy in the engine's type
+        wanted_behind = low and isinstance(next_norm, StreamCopyWanted)
+        h = x
+        if low:
+            h = prepared if isinstance(prepared, torch.Tensor) else ops.cast_rows(x, self._copy(x))
+        y = self.mixer.forward(h, ctx, caches.get("mixer"), states.get("mixer"), None)
+        second = self.ffn_norm is not None
+        copy = self._copy(x) if low and (self.ffn is not None or (not second and wanted_behind)) else None
+        self.mixer_norm.sum_normed(y, x, self.alpha, copy)
+        if not second:
+            return x, copy
+        y = self.ffn.forward(copy if low else x, ctx, None) if self.ffn is not None else None
+        copy = self._copy(x) if wanted_behind else None
+        self.ffn_norm.sum_normed(y, x, self.alpha, copy)
+        return x, copy
+
+
 register_block("pre_norm", PreNormBlock)
+register_block("sum_norm", SumNormBlock)
 register_block("output_norm", OutputNormBlock)

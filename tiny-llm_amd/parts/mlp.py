@@ -100,5 +100,45 @@ class ClampedGLU(FeedForward):
         return ops.linear(z, self.w_down, residual, residual)
 
 
+class GeluGLU(FeedForward):
+    """down(gelu(gate(h)) * up(h)), gelu in its tanh form.  Gate and up weights are stacked on load into
+    one [2F, H] matrix (one product); the activation runs on its result in the engine's element type.
+    `names`: the tensors' names below the prefix, (gate, up, down).  With `residual=None` the result is
+    returned by itself in float32."""
+    graph_safe = True
+
+    def __init__(self, prefix, dtype, device, *, hidden_size: int, intermediate_size: int,
+                 names=("gate", "up", "down")):
+        super().__init__(prefix, dtype, device)
+        self.hidden_size = int(hidden_size)
+        self.intermediate_size = int(intermediate_size)
+        ops.check_linear_sizes(dtype, self.hidden_size, f"{prefix}: hidden_size")
+        ops.check_linear_sizes(dtype, self.intermediate_size, f"{prefix}: intermediate_size")
+        self.names = tuple(f"{prefix}.{n}" for n in names)
+        self.w_gate_up: Optional[torch.Tensor] = None
+        self.w_down: Optional[torch.Tensor] = None
+
+    def weights(self) -> List[WeightSpec]:
+        H, I = self.hidden_size, self.intermediate_size
+        gate, up, down = self.names
+        return [WeightSpec(gate, (I, H)), WeightSpec(up, (I, H)), WeightSpec(down, (H, I))]
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        gate, up, down = self.names
+        self.w_gate_up = torch.cat([tensors[gate], tensors[up]], dim=0).contiguous()
+        self.w_down = tensors[down].contiguous()
+
+    def forward(self, h, ctx, residual):
+        T, dev = h.shape[0], h.device
+        gu = ops.scratch("ffn_gate_up", (T, 2 * self.intermediate_size), self.dtype, dev)
+        ops.linear(h, self.w_gate_up, gu)
+        z = ops.scratch("ffn_gated", (T, self.intermediate_size), self.dtype, dev)
+        ops.gelu_glu(gu, z)
+        if residual is None:
+            return ops.linear(z, self.w_down, ops.scratch("sublayer_out", (T, self.hidden_size), torch.float32, dev))
+        return ops.linear(z, self.w_down, residual, residual)
+
+
 register_feed_forward("swiglu", SwiGLU)
+register_feed_forward("gelu_glu", GeluGLU)
 register_feed_forward("clamped_glu", ClampedGLU)

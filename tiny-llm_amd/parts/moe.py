@@ -1,0 +1,93 @@
+"""A mixture of small gated feed-forward layers without a router: a table gives every token id its
+`top` experts, each with weight 1 / top; an optional shared expert runs for every token and is added,
+optionally times sigmoid(w_sg . h), one number per token.
+
+Experts are `clamped_glu` units (parts/mlp.py): down(g * sigmoid(alpha g) * (u + shift)) with
+g = min(gate(h), limit), u = clamp(up(h), -limit, limit), without biases.  Their weights are stacked on
+load ([E, 2F, W] and [E, W, F]); a step multiplies every token's row with the weights of its own experts.
+Tensor names below the prefix: e<i>.gate|up|down, table, shared.gate|up|down, shared.sg.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional
+
+import torch
+
+from ..kernels import ops
+from .base import FeedForward, WeightSpec, add_to_residual, register_feed_forward
+from .mlp import ClampedGLU
+
+
+class TableMoE(FeedForward):
+    graph_safe = True
+
+    def __init__(self, prefix, dtype, device, *, hidden_size: int, vocab_size: int, num_experts: int, top: int,
+                 intermediate_size: int, limit: float, alpha: float = 1.702, shift: float = 1.0,
+                 shared: Optional[dict] = None):
+        """shared: None, or {"intermediate_size": F, "limit": L, "gate": bool} for the shared expert."""
+        super().__init__(prefix, dtype, device)
+        self.hidden_size, self.vocab_size = int(hidden_size), int(vocab_size)
+        self.num_experts, self.top, self.intermediate_size = int(num_experts), int(top), int(intermediate_size)
+        self.limit, self.alpha, self.shift = float(limit), float(alpha), float(shift)
+        if not (0 < self.top <= self.num_experts):
+            raise ValueError(f"{prefix}: a token uses 1 to {self.num_experts} experts, got top = {self.top}")
+        if not self.limit > 0:
+            raise ValueError(f"{prefix}: the limit of the gated unit must be positive")
+        ops.check_linear_sizes(dtype, self.hidden_size, f"{prefix}: hidden_size")
+        ops.check_linear_sizes(dtype, self.intermediate_size, f"{prefix}: expert intermediate_size")
+        self.shared = None
+        self.shared_gate = False
+        if shared:
+            self.shared = ClampedGLU(f"{prefix}.shared", dtype, device, hidden_size=self.hidden_size,
+                                     intermediate_size=int(shared["intermediate_size"]), limit=float(shared["limit"]),
+                                     alpha=float(shared.get("alpha", alpha)), shift=float(shared.get("shift", shift)))
+            self.shared_gate = bool(shared.get("gate", True))
+        self.w_gate_up = self.w_down = self.table = self.w_sg = None
+
+    def weights(self) -> List[WeightSpec]:
+        p, W, F = self.prefix, self.hidden_size, self.intermediate_size
+        out = []
+        for e in range(self.num_experts):
+            out += [WeightSpec(f"{p}.e{e}.gate", (F, W)), WeightSpec(f"{p}.e{e}.up", (F, W)),
+                    WeightSpec(f"{p}.e{e}.down", (W, F))]
+        out.append(WeightSpec(f"{p}.table", (self.vocab_size, self.top), role="table", init=f"distinct:{self.num_experts}"))
+        if self.shared is not None:
+            out += self.shared.weights()
+            if self.shared_gate:
+                out.append(WeightSpec(f"{p}.shared.sg", (1, W)))
+        return out
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        p, E = self.prefix, self.num_experts
+        self.w_gate_up = torch.stack([torch.cat([tensors[f"{p}.e{e}.gate"], tensors[f"{p}.e{e}.up"]], dim=0)
+                                      for e in range(E)]).contiguous()
+        self.w_down = torch.stack([tensors[f"{p}.e{e}.down"] for e in range(E)]).contiguous()
+        table = tensors[f"{p}.table"].to(torch.int32).contiguous()
+        if table.numel() and (int(table.min()) < 0 or int(table.max()) >= E):
+            raise ValueError(f"{p}.table names experts outside 0 .. {E - 1}")
+        self.table = table
+        if self.shared is not None:
+            self.shared.bind(tensors)
+            if self.shared_gate:
+                self.w_sg = tensors[f"{p}.shared.sg"].reshape(-1).contiguous()
+
+    def forward(self, h, ctx, residual):
+        T, dev, F = h.shape[0], h.device, self.intermediate_size
+        tokens = ctx.tokens
+        base = scale = None
+        if self.shared is not None:
+            base = self.shared.forward(h, ctx, None)
+            if self.shared_gate:
+                scale = ops.row_dot_sigmoid(h, self.w_sg, ops.scratch("moe_shared_gate", (T,), torch.float32, dev))
+        gu = ops.scratch("moe_gate_up", (T * self.top, 2 * F), self.dtype, dev)
+        ops.table_moe_up(h, self.w_gate_up, tokens, self.table, gu)
+        z = ops.scratch("moe_gated", (T * self.top, F), self.dtype, dev)
+        ops.clamped_glu(gu, z, self.limit, self.alpha, self.shift)
+        out = base if base is not None else ops.scratch("sublayer_out", (T, self.hidden_size), torch.float32, dev)
+        ops.table_moe_down(z, self.w_down, tokens, self.table, out, 1.0 / self.top, base, scale)
+        if residual is None:
+            return out
+        return add_to_residual(residual, out)
+
+
+register_feed_forward("table_moe", TableMoE)

@@ -115,6 +115,46 @@ class RMSNorm(Norm):
         return ops.rmsnorm(x, self.weight, self.eps, out, rows)
 
 
+class LayerNorm(Norm):
+    """(x - mean) / sqrt(var + eps) * w + b over a row, var the mean squared deviation; statistics, weight
+    and bias in float32.  `weight_name` / `bias_name`: the tensors' names below the prefix ("" for the
+    prefix itself).  `sum_normed` serves a layer whose norm FOLLOWS the sum: x <- LN(alpha * x + y)."""
+    graph_safe = True
+
+    def __init__(self, prefix, dtype, device, *, hidden_size: int, eps: float, weight_name: str = "weight",
+                 bias_name: str = "bias"):
+        super().__init__(prefix, dtype, device)
+        self.hidden_size = int(hidden_size)
+        self.eps = float(eps)
+        if not self.eps > 0:
+            raise ValueError(f"{prefix}: eps must be positive")
+        self.weight_name = f"{prefix}.{weight_name}" if weight_name else prefix
+        self.bias_name = f"{prefix}.{bias_name}" if bias_name else prefix
+        if self.weight_name == self.bias_name:
+            raise ValueError(f"{prefix}: weight and bias need two tensor names")
+        self.weight: Optional[torch.Tensor] = None
+        self.bias: Optional[torch.Tensor] = None
+
+    def weights(self) -> List[WeightSpec]:
+        return [WeightSpec(self.weight_name, (self.hidden_size,), role="vector", init="ones"),
+                WeightSpec(self.bias_name, (self.hidden_size,), role="vector", init="zeros")]
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        self.weight = tensors[self.weight_name].to(torch.float32).contiguous()
+        self.bias = tensors[self.bias_name].to(torch.float32).contiguous()
+
+    def sum_normed(self, y: Optional[torch.Tensor], x: torch.Tensor, alpha: float,
+                   copy: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """x <- LN(alpha * x + y) in place (y float32 or None, one kernel); `copy` receives the new x in
+        its own element type."""
+        return ops.layer_norm_sum(y, self.weight, self.bias, x, alpha, self.eps, copy)
+
+    def forward(self, x: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        n = x.shape[0] if rows is None else rows.numel()
+        out = ops.scratch("normed", (n, self.hidden_size), self.dtype, x.device, rotate=2)
+        return ops.layer_norm_rows(x, self.weight, self.bias, self.eps, out, rows)
+
+
 class VectorScale(ChannelScale):
     """A learned vector that multiplies a sublayer's result channel by channel; kept in float32.
     The tensor is named by the prefix itself."""
@@ -133,4 +173,5 @@ class VectorScale(ChannelScale):
 
 
 register_norm("rmsnorm", RMSNorm)
+register_norm("layernorm", LayerNorm)
 register_scale("vector", VectorScale)

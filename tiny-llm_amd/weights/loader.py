@@ -296,6 +296,13 @@ def random_tensor(spec: WeightSpec, seed: int, std: float, norm_std: float, devi
     """The tensor that (seed, name) stands for, float32 rounded to `dtype`; independent of load
     order, and the same bits whether it is made on the host or on a GPU."""
     if spec.role == "table":
+        if spec.init.startswith("distinct:"):
+            # rows of distinct numbers below n: a start that depends on the row (and the seed), then its successors
+            n = int(spec.init.split(":", 1)[1])
+            rows, cols = spec.shape
+            start = (torch.arange(rows, dtype=torch.int64) * 2654435761 + tensor_key(seed, spec.name) % 1000003) % n
+            t = (start[:, None] + torch.arange(cols, dtype=torch.int64)[None, :]) % n
+            return t.to(torch.int32).to(device)
         return torch.zeros(spec.shape, dtype=torch.int32, device=device)
     scale, shift = _scale_and_shift(spec, std, norm_std)
     n = int(np.prod(spec.shape, dtype=np.int64)) if spec.shape else 1
