@@ -138,7 +138,7 @@ def clamped_expert(h, w, limit):
 
 def table_moe(h, w, mlp, tokens):
     """Every token's experts come from a table row of its id; each weighs 1 / top.  A shared
-    expert, if the layer has one, is added times sigmoid(w_sg . h)."""
+    expert, if the layer has one, is added, times sigmoid(w_sg . h) if it has a gate."""
     top = mlp["router"]["top"]
     table = w["table"].to(torch.long)
     out = torch.zeros_like(h)
@@ -147,7 +147,8 @@ def table_moe(h, w, mlp, tokens):
             out[t] += clamped_expert(h[t:t + 1], _sub(w, f"e{e}."), mlp["expert"]["limit"])[0] / top
     if mlp.get("shared"):
         s = _sub(w, "shared.")
-        out = out + clamped_expert(h, s, mlp["shared"]["limit"]) * torch.sigmoid(h @ s["sg"].T)
+        y = clamped_expert(h, s, mlp["shared"]["limit"])
+        out = out + (y * torch.sigmoid(h @ s["sg"].T) if "sg" in s else y)
     return out
 
 
@@ -168,6 +169,8 @@ def layer_forward(cfg, w, i: int, x, tokens, positions):
         mw = _sub(lw, "mlp.")
         y = dense_ff(x, mw) if mlp["kind"] == "dense" else table_moe(x, mw, mlp, tokens)
         x = layer_norm(alpha * x + y, lw["norm2"], lw["norm2.b"], eps)
+    elif "norm2" in lw:                                   # no feed-forward, but the second norm is there
+        x = layer_norm(alpha * x, lw["norm2"], lw["norm2.b"], eps)
     return x
 
 

@@ -1,0 +1,116 @@
+"""The Fofapel configuration reader and model spec (no GPU): sizes from config.json keys and from tensor
+shapes, refusals by name, the spec's tensors against the test checkpoints', cache groups and state rows; and
+properties of the plain implementation that a misread equation would break."""
+import copy
+
+import pytest
+import torch
+
+import plain_fofapel as plain
+from fofapel_util import CONFIGS, MIX_A, MIX_B, as_double, random_weights
+from tiny_llm_amd.config import ConfigError, FofapelConfig, resolve
+from tiny_llm_amd.models.decoder import Decoder
+
+
+@pytest.mark.parametrize("name", sorted(CONFIGS))
+def test_spec_names_the_checkpoints_tensors(name):
+    cfg, _ = CONFIGS[name]
+    w = random_weights(cfg, 1)
+    shapes = {k: tuple(v.shape) for k, v in w.items()}
+    stripped = copy.deepcopy(cfg)
+    for l in stripped["layers"]:
+        l.pop("norm2", None)
+        l["mixer"]["right"].pop("decay_rank", None)
+    for raw, given in ((cfg, None), (stripped, shapes)):
+        typed, spec = resolve(raw, given)
+        dec = Decoder(spec, dtype="bfloat16", device="cpu")
+        assert {s.name: tuple(s.shape) for s in dec.weight_specs()} == shapes
+        assert spec.architecture == "Fofapel" and len(spec.plan) == len(cfg["layers"])
+        assert all(s.role == "table" for s in dec.weight_specs() if s.name.endswith(".table"))
+    assert isinstance(typed, FofapelConfig)
+
+
+def test_sizes_that_only_the_tensors_know():
+    w = random_weights(MIX_B, 1)
+    shapes = {k: tuple(v.shape) for k, v in w.items()}
+    raw = copy.deepcopy(MIX_B)
+    for l in raw["layers"]:
+        l.pop("norm2", None)
+        l["mixer"]["right"]["decay_rank"] = 999            # the tensor's shape wins over a key
+    typed, _ = resolve(raw, shapes)
+    assert [l.mixer.right.decay_rank for l in typed.layers] == [16, 24, 8, 12]
+    assert [l.second_norm for l in typed.layers] == [True, True, True, True]
+    assert typed.layers[2].mlp is None
+    assert typed.layers[1].mlp.shared.gate is False and typed.layers[3].mlp.shared.gate is True
+    typed_a, _ = resolve(MIX_A)
+    assert [l.second_norm for l in typed_a.layers] == [True, True, False, True]
+
+
+def test_cache_groups_and_state_rows():
+    _, spec = resolve(MIX_A)
+    dec = Decoder(spec, dtype="float32", device="cpu")
+    caches = dec.cache_specs()
+    assert [caches[(i, "mixer")].window for i in range(4)] == [24, 7, 1000, 33]
+    assert all(c.kind == "window" and [t.name for t in c.tensors] == ["k", "v"] for c in caches.values())
+    states = dec.state_specs()
+    # S in slices of 16 key channels (24 -> 32, 80 -> 128) plus the last token's input
+    assert states[(0, "mixer")].shape == (2 * 32 * 24 + 64,)
+    assert states[(1, "mixer")].shape == (1 * 128 * 80 + 64,)
+    assert states[(2, "mixer")].shape == (3 * 16 * 16 + 64,)
+
+
+@pytest.mark.parametrize("change,message", [
+    (lambda c: c["layers"][0].update(type="serial"), "not built"),
+    (lambda c: c["layers"][0]["mlp"].update(kind="routed"), "not built"),
+    (lambda c: c["layers"][0]["mixer"]["left"].update(vdim=8), "values are the keys"),
+    (lambda c: c["layers"][0]["mixer"]["left"].update(kv_heads=3), "multiple"),
+    (lambda c: c["layers"][0]["mixer"]["left"]["rot"].update(dims=18), "rot.dims"),
+    (lambda c: c["layers"][0]["mlp"]["router"].update(top=9), "top"),
+    (lambda c: c.pop("postln_alpha"), "postln_alpha"),
+    (lambda c: c["layers"][1]["mixer"].pop("right"), "right"),
+])
+def test_refusals(change, message):
+    cfg = copy.deepcopy(MIX_A)
+    change(cfg)
+    with pytest.raises(ConfigError, match=message):
+        resolve(cfg)
+
+
+def test_sink_takes_weight_and_window_hides_keys():
+    s = torch.tensor([[0.3, -1.0, 2.0, 0.5]], dtype=torch.float64)
+    seen = torch.tensor([[True, True, False, True]])
+    p = plain.sink_softmax(s, seen)
+    e = torch.exp(s[0, [0, 1, 3]])
+    assert torch.allclose(p[0, [0, 1, 3]], e / (1.0 + e.sum())) and p[0, 2] == 0 and p.sum() < 1
+    big = plain.sink_softmax(torch.tensor([[800.0, 790.0]], dtype=torch.float64), torch.ones(1, 2, dtype=torch.bool))
+    assert torch.isfinite(big).all() and abs(float(big.sum()) - 1.0) < 1e-12
+
+
+def test_a_token_outside_every_window_reaches_the_logits_only_through_the_state():
+    """One layer: changing the first token moves the last row only through the time mix; with the time mix
+    switched off (right_scale 0) the last row does not move at all once the window has passed."""
+    cfg = copy.deepcopy(CONFIGS["dense"][0])
+    w = as_double(random_weights(cfg, 4))
+    a = list(range(1, 41))
+    b = [77] + a[1:]
+    assert (plain.forward(cfg, w, a)[-1] - plain.forward(cfg, w, b)[-1]).abs().max() > 1e-6
+    cfg["layers"][0]["mixer"]["right_scale"] = 0.0
+    assert (plain.forward(cfg, w, a)[-1] - plain.forward(cfg, w, b)[-1]).abs().max() == 0
+    assert (plain.forward(cfg, w, a)[19] - plain.forward(cfg, w, b)[19]).abs().max() > 1e-9     # inside the window of 20
+
+
+def test_recurrence_in_two_halves_equals_the_whole():
+    g = torch.Generator().manual_seed(0)
+    T, H, D = 12, 2, 5
+    r, k, v = (torch.randn(T, H, D, generator=g, dtype=torch.float64) for _ in range(3))
+    dec = torch.rand(T, H, D, generator=g, dtype=torch.float64)
+    u = torch.randn(H, D, generator=g, dtype=torch.float64)
+    whole = plain.time_mix_recurrence(r, k, v, dec, u)
+    # o_t by its closed form: sum over earlier tokens of the decayed outer products, plus the bonus term
+    for t in (0, 5, 11):
+        want = torch.zeros(H, D, dtype=torch.float64)
+        for j in range(t):
+            decay = torch.prod(dec[j + 1:t], dim=0) if t - j > 1 else torch.ones(H, D, dtype=torch.float64)
+            want += ((r[t] * decay * k[j]).sum(-1, keepdim=True)) * v[j]
+        want += ((r[t] * u * k[t]).sum(-1, keepdim=True)) * v[t]
+        assert torch.allclose(whole[t], want, atol=1e-12)
