@@ -13,7 +13,7 @@ Llama-3-8B shape; 64 requests of 1,024 tokens that nearly fill the cache at the 
 `--only` picks a part (for profiling), or one of the measurements that are not part of the line:
 `attention` (the attention kernels alone at contexts up to 131,072 tokens), `long_context` (the Llama-3-8B
 shape with 8 requests of 32,000 tokens and one of 131,000), `decode_shapes` (decode steps at the two larger
-shapes by batch), `host` (a step's wall time against its time on the GPU), `lufazen` (the Lufazen design,
+shapes by batch), `host` (a step's wall time against its time on the GPU), `fofapel` (the Fofapel design, as `lufazen`), `lufazen` (the Lufazen design,
 recurrent and latent-attention layers, at two sizes beside a Llama of equal size: prefill, decode, time by kernel).
 """
 import argparse
@@ -751,6 +751,68 @@ def lufazen_figures(args):
     Lufazen design at two sizes, each beside a Llama with the same number of layers, width, feed-forward
     size, heads of 128 and vocabulary; time by kernel for both; and for the kernels that only the new
     design has, what the published peaks would allow (bytes over 8 TB/s or flops over the matrix peak)."""
+    def bounds(dtype, heads, width, ff):
+        e = ELT[dtype]
+        T, ctx, B = PREFILL_TOKENS, PROMPT_LEN, 8
+        kr, rot = 512, 64
+        return {
+            "latent_attention prefill (flops of scores and values over the latent, causal)":
+                round(2.0 * heads * (T * T / 2) * (2 * kr + rot) / (PEAK_TFLOPS[dtype] * 1e12) * 1e6, 1),
+            "latent_attention decode b8 (the cached latents once)":
+                round(B * ctx * (kr + rot) * e / (HBM_GBS * 1e9) * 1e6, 2),
+            "delta_recurrence decode b8 (the states read and written)":
+                round(2.0 * B * heads * 128 * 128 * 4 / (HBM_GBS * 1e9) * 1e6, 2),
+            "delta_recurrence prefill (6 flops per state element and token, float32 vector units at 157 TFLOP/s)":
+                round(6.0 * T * heads * 128 * 128 / (157.3e12) * 1e6, 1),
+        }
+    return design_beside_llama(args, "lufazen", lufazen_config, bounds)
+
+
+def fofapel_config(layers, width, ff, heads, vocab=32000, window=512):
+    """Every layer: attention in a window of 512 tokens (heads of 128, four query heads a kv head) beside a
+    time mix of width / 64 heads of 64 channels (decay rank 64).  Feed-forwards in the order dense, experts,
+    experts, experts: the dense one of size ff; 8 experts of ff / 4, two a token, and a gated shared expert of
+    ff / 4 (three quarters of a dense layer's arithmetic a token)."""
+    out = []
+    for i in range(layers):
+        if i % 4 == 0:
+            mlp = {"kind": "dense", "ff": ff}
+        else:
+            mlp = {"kind": "moe", "router": {"experts": 8, "top": 2}, "expert": {"ff": ff // 4, "limit": 7.0},
+                   "shared": {"ff": ff // 4, "limit": 7.0}}
+        mixer = {"left": {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 128, "vdim": 128, "mask": {"size": window},
+                          "rot": {"base": 10000.0, "dims": 128}, "scale": 128 ** -0.5},
+                 "right": {"heads": width // 64, "dim": 64, "decay_rank": 64}, "left_scale": 1.0, "right_scale": 1.0}
+        out.append({"type": "parallel", "mixer": mixer, "mlp": mlp})
+    return {"architecture": "Fofapel", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "postln_alpha": 1.0,
+            "layers": out, "max_position": 8192}
+
+
+def fofapel_figures(args):
+    """The Fofapel design at two sizes beside a Llama of equal layers, width, feed-forward size, heads of 128 and
+    vocabulary, as `lufazen_figures`; bounds for the kernels that only this design has."""
+    def bounds(dtype, heads, width, ff):
+        e = ELT[dtype]
+        T, ctx, B, win = PREFILL_TOKENS, PROMPT_LEN, 8, 512
+        th = width // 64
+        return {
+            "window attention prefill (flops of scores and values inside the window)":
+                round(2.0 * heads * T * min(win, T / 2) * 2 * 128 / (PEAK_TFLOPS[dtype] * 1e12) * 1e6, 1),
+            "window attention decode b8 (the cached keys and values of the window once)":
+                round(B * min(ctx, win) * 2 * (heads // 4) * 128 * e / (HBM_GBS * 1e9) * 1e6, 2),
+            "time_mix_recurrence decode b8 (the states read and written)":
+                round(2.0 * B * th * 64 * 64 * 4 / (HBM_GBS * 1e9) * 1e6, 2),
+            "time_mix_recurrence prefill (5 flops per state element and token, float32 vector units at 157 TFLOP/s)":
+                round(5.0 * T * th * 64 * 64 / (157.3e12) * 1e6, 1),
+            "experts decode b8 (the weights of 16 experts' worth of rows at most: all 8 experts once)":
+                round(8 * 3 * width * (ff // 4) * e / (HBM_GBS * 1e9) * 1e6, 2),
+            "experts prefill (flops of two experts a token)":
+                round(2.0 * T * 2 * 3 * width * (ff // 4) / (PEAK_TFLOPS[dtype] * 1e12) * 1e6, 1),
+        }
+    return design_beside_llama(args, "fofapel", fofapel_config, bounds)
+
+
+def design_beside_llama(args, design, config_of, bounds_of):
     import torch
     dtype = args.dtype
     out = {}
@@ -758,7 +820,7 @@ def lufazen_figures(args):
         if args.layers:
             layers = args.layers
         row = {"layers": layers, "width": width, "ff": ff, "heads": heads}
-        for which, cfg in (("lufazen", lufazen_config(layers, width, ff, heads)),
+        for which, cfg in ((design, config_of(layers, width, ff, heads)),
                            ("llama", llama(layers, width, heads, heads, ff, 32000, 10000.0, 8192))):
             b = Bench(cfg, dtype, max_batch=8, total_new=args.steps + args.warmup + 200, block_size=args.block_size)
             r = {}
@@ -791,19 +853,7 @@ def lufazen_figures(args):
             b.close()
             row[which] = r
         # what the peaks allow for the new design's own kernels, per layer of that kind
-        e = ELT[dtype]
-        T, ctx, B = PREFILL_TOKENS, PROMPT_LEN, 8
-        kr, rot = 512, 64
-        row["bounds_us"] = {
-            "latent_attention prefill (flops of scores and values over the latent, causal)":
-                round(2.0 * heads * (T * T / 2) * (2 * kr + rot) / (PEAK_TFLOPS[dtype] * 1e12) * 1e6, 1),
-            "latent_attention decode b8 (the cached latents once)":
-                round(B * ctx * (kr + rot) * e / (HBM_GBS * 1e9) * 1e6, 2),
-            "delta_recurrence decode b8 (the states read and written)":
-                round(2.0 * B * heads * 128 * 128 * 4 / (HBM_GBS * 1e9) * 1e6, 2),
-            "delta_recurrence prefill (6 flops per state element and token, float32 vector units at 157 TFLOP/s)":
-                round(6.0 * T * heads * 128 * 128 / (157.3e12) * 1e6, 1),
-        }
+        row["bounds_us"] = bounds_of(dtype, heads, width, ff)
         out[name] = row
         print(json.dumps({name: row}), file=sys.stderr, flush=True)
     return out
@@ -812,6 +862,9 @@ def lufazen_figures(args):
 def run(args):
     if args.only == "lufazen":
         print(json.dumps({"lufazen_beside_llama": lufazen_figures(args)}), flush=True)
+        return
+    if args.only == "fofapel":
+        print(json.dumps({"fofapel_beside_llama": fofapel_figures(args)}), flush=True)
         return
     if args.only == "attention":
         print(json.dumps({"decode_attention": attention_sweep()}), flush=True)
@@ -888,14 +941,15 @@ def main():
     ap.add_argument("--block-size", type=int, default=16)
     ap.add_argument("--only", default="all",
                     choices=["all", "headline", "decode", "prefill", "fp32", "kernels", "peaks", "llama3_8b", "llama3_8b_prefill", "llama2_13b", "host",
-                             "attention", "long_context", "decode_shapes", "lufazen"],
+                             "attention", "long_context", "decode_shapes", "lufazen", "fofapel"],
                     help="all: everything in one line; headline: the bfloat16 TinyLlama figures only; decode / prefill: "
                          "one of them (profiling); fp32: the float32 figures as the headline; kernels: decode with the time of "
                          "a step by kernel (torch's profiler); peaks / llama3_8b / "
                          "llama2_13b: that part alone; host: a step's wall time against its time on the GPU; attention: the "
                          "attention kernels alone at contexts up to 131,072 tokens; long_context: the Llama-3-8B shape with "
                          "8 requests of 32,000 tokens and one of 131,000; decode_shapes: decode steps at the two larger shapes by batch; "
-                         "lufazen: prefill and decode of the Lufazen design at two sizes beside a Llama of equal size, by kernel")
+                         "lufazen: prefill and decode of the Lufazen design at two sizes beside a Llama of equal size, by kernel; "
+                         "fofapel: the same for the Fofapel design")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         if int(os.environ.get("RANK", "0")) == 0:

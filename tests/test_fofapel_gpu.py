@@ -258,7 +258,9 @@ def _paged_kv(rows: torch.Tensor, table, block, n_blocks, dtype):
     return pages
 
 
-ATTENTION_KERNELS = ["general float32", "general bfloat16"]
+ATTENTION_KERNELS = ["general float32", "general bfloat16", "matrix cores float32", "matrix cores float32, chunks",
+                     "matrix cores float32, many rows", "matrix cores bfloat16", "matrix cores bfloat16, split keys",
+                     "matrix cores bfloat16, prompt", "matrix cores bfloat16, prompt, split keys"]
 
 
 @pytest.mark.parametrize("kernel", ATTENTION_KERNELS)
@@ -301,8 +303,36 @@ def test_window_and_sink_find_one_key(kernel, window):
     bt = torch.tensor([table + [0] * (64 - len(table))], dtype=torch.int32, device="cuda")
     out = torch.empty(T, heads * d, dtype=dtype, device="cuda")
     qd = q.reshape(T, heads * d).to(dtype).cuda()
-    ops.paged_attention(qd, k_pages, v_pages, bt, torch.zeros(T, dtype=torch.int32, device="cuda"), pos_dev, out,
-                        heads, kvh, d, 1.0, window, sink=True)
+    each = torch.arange(T, dtype=torch.int32, device="cuda")
+    tables = bt.repeat(T, 1).contiguous()         # every query a request of its own over the same pages
+    if kernel.startswith("general"):
+        ops.paged_attention(qd, k_pages, v_pages, bt, torch.zeros(T, dtype=torch.int32, device="cuda"), pos_dev, out,
+                            heads, kvh, d, 1.0, window, sink=True)
+    elif "float32" in kernel and "many rows" in kernel:
+        # a thousand query tiles and more: the kernel that gives a wave a tile
+        reps = -(-1024 // (T * kvh)) + 1
+        big = torch.empty(T * reps, heads * d, dtype=dtype, device="cuda")
+        n_t = T * reps
+        tiles = (torch.arange(n_t, dtype=torch.int32, device="cuda"),) * 2 + (torch.ones(n_t, dtype=torch.int32, device="cuda"),)
+        ops.attention_f32(qd.repeat(reps, 1), k_pages, v_pages, bt.repeat(n_t, 1).contiguous(), tiles, pos_dev.repeat(reps),
+                          big, heads, kvh, d, 1.0, window, sink=True)
+        assert all(torch.equal(big[:T], big[r * T:(r + 1) * T]) for r in range(1, reps))
+        out = big[:T]
+    elif "float32" in kernel:
+        chunks = -(-700 // ops.F32_CHUNK_KEYS) if "chunks" in kernel else 1
+        part = torch.empty(chunks * T * heads * (d + 2), device="cuda") if chunks > 1 else None
+        ops.attention_f32(qd, k_pages, v_pages, tables, None, pos_dev, out, heads, kvh, d, 1.0, window, chunks, part,
+                          sink=True)
+    elif "prompt" in kernel:
+        splits = 3 if "split" in kernel else 1
+        part = torch.empty(splits * T * heads * (d + 2), device="cuda") if splits > 1 else None
+        ops.flash_prefill(qd, k_pages, v_pages, tables, (each, each.clone(), torch.ones_like(each)), pos_dev, out, heads, kvh,
+                          d, 1.0, window, 4, splits, part, sink=True)
+    else:
+        splits = 3 if "split" in kernel else 1
+        part = torch.empty(splits * T * heads * (d + 2), device="cuda") if splits > 1 else None
+        ops.flash_attention(qd, k_pages, v_pages, tables, None, pos_dev, out, heads, kvh, d, 1.0, window, splits, part,
+                            sink=True)
     kr, vr, qr = keys.to(dtype).double(), vals.to(dtype).double(), q.to(dtype).double()
     out = out.double().cpu().reshape(T, heads, d)
     for i, pos in enumerate(positions):

@@ -40,7 +40,7 @@ def call(lib, static, batch, nq, nkv, hd, bs, n_splits, out, scratch=None):
     stream = c_void_p(torch.cuda.current_stream().cuda_stream)
     head = (ptr(q), c_int64(q.stride(0)), ptr(k), ptr(v), ptr(bt), c_int(bt.shape[1]), ptr(None), ptr(None), ptr(None),
             ptr(pos), ptr(out), c_int64(out.stride(0)))
-    tail = (c_int(T), c_int(T), c_int(nq), c_int(nkv), c_int(hd), c_int(bs), c_float(hd ** -0.5), c_int(0),
+    tail = (c_int(T), c_int(T), c_int(nq), c_int(nkv), c_int(hd), c_int(bs), c_float(hd ** -0.5), c_int(0), c_int(0),
             c_int(n_splits), ptr(None), ptr(None), c_int(0), stream)
     if static:
         return lib.tl_flash_attention_static(*head, *tail)

@@ -118,6 +118,13 @@ constexpr int FA_KT = 64;
 constexpr int FA_VPAD = 8;      // padding of a row of the row-major V tile in LDS (elements)
 constexpr float kNegBig = -1.0e30f;   // "no key yet": finite, so exp2(m - m') never sees inf - inf
 
+// A sink: one more term in the softmax's denominator, with score 0 and no value.  l is the sum of
+// exp2(s - m) over the keys, m in units of log2 e; the term is exp2(0 - m) (infinite for a very negative m,
+// which makes the result the zero it then is).
+__device__ __forceinline__ float with_sink(float l, float m, int sink) {
+  return sink ? l + __builtin_amdgcn_exp2f(-m) : l;
+}
+
 // Two probabilities as two bfloat16 terms each, p = hi + lo, packed pairwise.  hi is p with the low
 // 16 bits cut off (exact, one mask), lo = p - hi is exact in float32 and rounded to bfloat16: the
 // pair carries 16 bits of p, as rounding hi would, for three vector instructions a value
@@ -179,7 +186,7 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_attn_bf16_kernel(
     const int32_t* __restrict__ tile_req, const int32_t* __restrict__ tile_tok0,
     const int32_t* __restrict__ tile_ntok, const int32_t* __restrict__ positions, bf16_t* __restrict__ out,
     int64_t out_stride, float* __restrict__ part_o, float* __restrict__ part_ml, int nq, int nkv,
-    int block_size, float scale, int window, int n_splits, int n_tokens, const FusedRope fused) {
+    int block_size, float scale, int window, int sink, int n_splits, int n_tokens, const FusedRope fused) {
   constexpr int HD = HDT * 16;
   constexpr int KS = (HD + 31) / 32;       // k-steps of the score product
   constexpr int VS = HD + FA_VPAD;         // row stride of a wave's V tile in LDS
@@ -521,7 +528,8 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_attn_bf16_kernel(
       acc += wgt * area[d];
     }
     if (n_splits == 1) {
-      out[(int64_t)t * out_stride + (int64_t)h * HD + d] = (bf16_t)(L > 0.f ? acc / L : 0.f);
+      const float Ls = with_sink(L, M, sink);
+      out[(int64_t)t * out_stride + (int64_t)h * HD + d] = (bf16_t)(Ls > 0.f ? acc / Ls : 0.f);
     } else {
       part_o[(((int64_t)split * n_tokens + t) * nq + h) * HD + d] = acc;
       if (d == 0) {
@@ -699,7 +707,7 @@ __global__ __launch_bounds__(A32_THREADS) void attention_f32_kernel(
     const float* __restrict__ v_cache, const int32_t* __restrict__ block_tables, int max_blocks,
     const int32_t* __restrict__ tile_req, const int32_t* __restrict__ tile_tok0,
     const int32_t* __restrict__ tile_ntok, const int32_t* __restrict__ positions, float* __restrict__ out,
-    int64_t out_stride, float* __restrict__ part, int nq, int nkv, int block_size, float scale, int window,
+    int64_t out_stride, float* __restrict__ part, int nq, int nkv, int block_size, float scale, int window, int sink,
     int n_tokens) {
   constexpr int HD = HDT * 16;
   constexpr int PS = HD + 4;                       // row stride of a tile's O in LDS
@@ -790,7 +798,8 @@ __global__ __launch_bounds__(A32_THREADS) void attention_f32_kernel(
     if (t_local >= TW || t_local >= ntok) continue;
     const int t = tok0 + t_local, h = kvh * G + h_local;
     if (gridDim.z == 1) {
-      out[(int64_t)t * out_stride + (int64_t)h * HD + d] = Lrun[u] > 0.f ? Orun[u] / Lrun[u] : 0.f;
+      const float Ls = with_sink(Lrun[u], Mrun[u], sink);
+      out[(int64_t)t * out_stride + (int64_t)h * HD + d] = Ls > 0.f ? Orun[u] / Ls : 0.f;
     } else {
       float* pr = part + (((int64_t)blockIdx.z * n_tokens + t) * nq + h) * (HD + 2);
       pr[d] = Orun[u];
@@ -815,7 +824,7 @@ __global__ __launch_bounds__(A32_THREADS) void attention_f32_rows_kernel(
     const float* __restrict__ v_cache, const int32_t* __restrict__ block_tables, int max_blocks,
     const int32_t* __restrict__ tile_req, const int32_t* __restrict__ tile_tok0,
     const int32_t* __restrict__ tile_ntok, const int32_t* __restrict__ positions, float* __restrict__ out,
-    int64_t out_stride, int nq, int nkv, int block_size, float scale, int window, int n_tiles) {
+    int64_t out_stride, int nq, int nkv, int block_size, float scale, int window, int sink, int n_tiles) {
   constexpr int HD = HDT * 16;
   extern __shared__ __attribute__((aligned(16))) float smem32[];
   const int tid = threadIdx.x, lane = tid % TL_WAVE, wave = tid / TL_WAVE;
@@ -879,10 +888,11 @@ __global__ __launch_bounds__(A32_THREADS) void attention_f32_rows_kernel(
   }
   if (!row_valid) return;
   float* orow = out + (int64_t)tok * out_stride + (int64_t)(kvh * G + hh) * HD;
+  const float Ls = with_sink(Lrun, Mrun, sink);
 #pragma unroll
   for (int dt = 0; dt < HDT; ++dt)
 #pragma unroll
-    for (int r = 0; r < 4; ++r) orow[dt * 16 + kk * 4 + r] = Lrun > 0.f ? Orun[dt][r] / Lrun : 0.f;
+    for (int r = 0; r < 4; ++r) orow[dt * 16 + kk * 4 + r] = Ls > 0.f ? Orun[dt][r] / Ls : 0.f;
 }
 
 // Merges the chunks that attention_f32_kernel left in `part` [chunks][tokens][heads][hd + 2], in
@@ -890,7 +900,8 @@ __global__ __launch_bounds__(A32_THREADS) void attention_f32_rows_kernel(
 // chunks itself.  One wave per (token, head).
 __global__ __launch_bounds__(TL_WAVE) void attention_f32_combine_kernel(const float* __restrict__ part,
                                                                        float* __restrict__ out, int64_t out_stride,
-                                                                       int n_tokens, int nq, int hd, int n_chunks) {
+                                                                       int n_tokens, int nq, int hd, int n_chunks,
+                                                                       int sink) {
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   for (int d = lane; d < hd; d += TL_WAVE) {
     float M = kNegBig, L = 0.f, O = 0.f, wa, wb;
@@ -899,7 +910,8 @@ __global__ __launch_bounds__(TL_WAVE) void attention_f32_combine_kernel(const fl
       merge_f32(M, L, pr[hd], pr[hd + 1], wa, wb);
       O = merge_f32_value(O, pr[d], wa, wb);
     }
-    out[(int64_t)t * out_stride + (int64_t)h * hd + d] = L > 0.f ? O / L : 0.f;
+    const float Ls = with_sink(L, M, sink);
+    out[(int64_t)t * out_stride + (int64_t)h * hd + d] = Ls > 0.f ? O / Ls : 0.f;
   }
 }
 
@@ -920,7 +932,7 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_prefill_bf16_kernel(
     const int32_t* __restrict__ tile_req, const int32_t* __restrict__ tile_tok0,
     const int32_t* __restrict__ tile_ntok, const int32_t* __restrict__ positions, bf16_t* __restrict__ out,
     int64_t out_stride, float* __restrict__ part_o, float* __restrict__ part_ml, int n_tiles, int n_tokens,
-    int n_splits, int nq, int nkv, int block_size, int bs_shift, float scale, int window) {
+    int n_splits, int nq, int nkv, int block_size, int bs_shift, float scale, int window, int sink) {
   constexpr int HD = HDT * 16;
   constexpr int KS = (HD + 31) / 32;
   constexpr int KP = KS * 32 + 8;
@@ -1237,7 +1249,8 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_prefill_bf16_kernel(
       }
       continue;
     }
-    const float inv = l > 0.f ? 1.f / l : 0.f;
+    const float ls = with_sink(l, m_run[rt], sink);
+    const float inv = ls > 0.f ? 1.f / ls : 0.f;
     bf16_t* orow = out + (int64_t)tok[rt] * out_stride + (int64_t)head * HD + g * 4;
 #pragma unroll
     for (int dt = 0; dt < HDT; ++dt) {
@@ -1257,7 +1270,7 @@ template <int FC_BATCH>
 __global__ __launch_bounds__(TL_WAVE) void flash_combine_kernel(const float* __restrict__ part_o,
                                                                 const float* __restrict__ part_ml,
                                                                 bf16_t* __restrict__ out, int64_t out_stride,
-                                                                int n_tokens, int nq, int hd, int n_splits) {
+                                                                int n_tokens, int nq, int hd, int n_splits, int sink) {
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int64_t row = (int64_t)t * nq + h, step = (int64_t)n_tokens * nq;      // split s: row + s * step
   // maxima are in units of log2 e; a split without keys has l = 0 and O = 0
@@ -1285,7 +1298,8 @@ __global__ __launch_bounds__(TL_WAVE) void flash_combine_kernel(const float* __r
           acc += wgt * o[u];
         }
       }
-      out[(int64_t)t * out_stride + (int64_t)h * hd + d] = (bf16_t)(L > 0.f ? acc / L : 0.f);
+      const float Ls = with_sink(L, M, sink);
+      out[(int64_t)t * out_stride + (int64_t)h * hd + d] = (bf16_t)(Ls > 0.f ? acc / Ls : 0.f);
     }
     return;
   }
@@ -1316,7 +1330,8 @@ __global__ __launch_bounds__(TL_WAVE) void flash_combine_kernel(const float* __r
         }
       }
     }
-    out[(int64_t)t * out_stride + (int64_t)h * hd + d] = (bf16_t)(L > 0.f ? acc / L : 0.f);
+    const float Ls = with_sink(L, M, sink);
+    out[(int64_t)t * out_stride + (int64_t)h * hd + d] = (bf16_t)(Ls > 0.f ? acc / Ls : 0.f);
   }
 }
 
@@ -1325,7 +1340,7 @@ static int launch_flash_w(const bf16_t* q, int64_t q_stride, const bf16_t* k_cac
                           const int32_t* block_tables, int max_blocks, const int32_t* tile_req,
                           const int32_t* tile_tok0, const int32_t* tile_ntok, const int32_t* positions, bf16_t* out,
                           int64_t out_stride, float* part_o, float* part_ml, int n_tiles, int n_tokens, int nq,
-                          int nkv, int block_size, float scale, int window, int n_splits, const FusedRope& fused,
+                          int nkv, int block_size, float scale, int window, int sink, int n_splits, const FusedRope& fused,
                           hipStream_t stream) {
   constexpr int HD = HDT * 16;
   constexpr size_t stage = (size_t)WAVES * FA_KT * (HD + FA_VPAD) * sizeof(bf16_t);
@@ -1340,7 +1355,7 @@ static int launch_flash_w(const bf16_t* q, int64_t q_stride, const bf16_t* k_cac
   }
   hipLaunchKernelGGL((flash_attn_bf16_kernel<HDT, WAVES>), dim3(n_tiles, nkv, n_splits), dim3(WAVES * TL_WAVE), stage,
                      stream, q, q_stride, k_cache, v_cache, block_tables, max_blocks, tile_req, tile_tok0, tile_ntok,
-                     positions, out, out_stride, part_o, part_ml, nq, nkv, block_size, scale, window, n_splits,
+                     positions, out, out_stride, part_o, part_ml, nq, nkv, block_size, scale, window, sink, n_splits,
                      n_tokens, fused);
   return TL_OK;
 }
@@ -1358,17 +1373,17 @@ static int launch_flash(const bf16_t* q, int64_t q_stride, const bf16_t* k_cache
                         const int32_t* block_tables, int max_blocks, const int32_t* tile_req,
                         const int32_t* tile_tok0, const int32_t* tile_ntok, const int32_t* positions, bf16_t* out,
                         int64_t out_stride, float* part_o, float* part_ml, int n_tiles, int n_tokens, int nq, int nkv,
-                        int block_size, float scale, int window, int n_splits, const FusedRope& fused,
+                        int block_size, float scale, int window, int sink, int n_splits, const FusedRope& fused,
                         hipStream_t stream) {
   if constexpr (HDT <= 4) {
     if (flash_waves(HDT * 16, n_tiles * nkv) == 8)
       return launch_flash_w<HDT, 8>(q, q_stride, k_cache, v_cache, block_tables, max_blocks, tile_req, tile_tok0,
                                     tile_ntok, positions, out, out_stride, part_o, part_ml, n_tiles, n_tokens, nq, nkv,
-                                    block_size, scale, window, n_splits, fused, stream);
+                                    block_size, scale, window, sink, n_splits, fused, stream);
   }
   return launch_flash_w<HDT, 4>(q, q_stride, k_cache, v_cache, block_tables, max_blocks, tile_req, tile_tok0, tile_ntok,
                                 positions, out, out_stride, part_o, part_ml, n_tiles, n_tokens, nq, nkv, block_size,
-                                scale, window, n_splits, fused, stream);
+                                scale, window, sink, n_splits, fused, stream);
 }
 
 }  // namespace
@@ -1408,7 +1423,7 @@ int tl_attention_f32(const float* q, int64_t q_stride, const float* k_cache, con
                      const int32_t* block_tables, int max_blocks, const int32_t* tile_req,
                      const int32_t* tile_tok0, const int32_t* tile_ntok, const int32_t* positions, float* out,
                      int64_t out_stride, float* part, int n_tiles, int n_tokens, int nq, int nkv, int hd,
-                     int block_size, float scale, int window, int n_chunks, hipStream_t stream) {
+                     int block_size, float scale, int window, int sink, int n_chunks, hipStream_t stream) {
   if (n_tiles <= 0 || n_tokens <= 0) return TL_OK;
   if (nq <= 0 || nkv <= 0 || nq % nkv || nq / nkv > 16 || hd <= 0 || hd % 16 || hd > 128 || block_size <= 0 ||
       max_blocks <= 0 || window < 0 || n_chunks < 1 || nkv > 65535 || n_chunks > 65535 || q_stride % 4 ||
@@ -1434,7 +1449,7 @@ int tl_attention_f32(const float* q, int64_t q_stride, const float* k_cache, con
     hipLaunchKernelGGL(attention_f32_rows_kernel<HDT>, dim3((n_tiles + A32_WAVES - 1) / A32_WAVES, nkv),           \
                        dim3(A32_THREADS), smem_rows, stream, q, q_stride, k_cache, v_cache, block_tables,          \
                        max_blocks, tile_req, tile_tok0, tile_ntok, positions, out, out_stride, nq, nkv,            \
-                       block_size, scale, window, n_tiles);                                                        \
+                       block_size, scale, window, sink, n_tiles);                                                        \
   } break;
     switch (hd / 16) {
       TL_A32_ROWS(1) TL_A32_ROWS(2) TL_A32_ROWS(3) TL_A32_ROWS(4)
@@ -1454,7 +1469,7 @@ int tl_attention_f32(const float* q, int64_t q_stride, const float* k_cache, con
     }                                                                                                             \
     hipLaunchKernelGGL(attention_f32_kernel<HDT>, dim3(n_tiles, nkv, n_chunks), dim3(A32_THREADS), smem, stream,  \
                        q, q_stride, k_cache, v_cache, block_tables, max_blocks, tile_req, tile_tok0, tile_ntok,   \
-                       positions, out, out_stride, part, nq, nkv, block_size, scale, window, n_tokens);           \
+                       positions, out, out_stride, part, nq, nkv, block_size, scale, window, sink, n_tokens);           \
   } break;
   switch (hd / 16) {
     TL_A32_CASE(1) TL_A32_CASE(2) TL_A32_CASE(3) TL_A32_CASE(4)
@@ -1463,7 +1478,7 @@ int tl_attention_f32(const float* q, int64_t q_stride, const float* k_cache, con
 #undef TL_A32_CASE
   if (n_chunks > 1)
     hipLaunchKernelGGL(attention_f32_combine_kernel, dim3(n_tokens, nq), dim3(TL_WAVE), 0, stream, part, out,
-                       out_stride, n_tokens, nq, hd, n_chunks);
+                       out_stride, n_tokens, nq, hd, n_chunks, sink);
   return tl_launch_status();
 }
 
@@ -1474,7 +1489,7 @@ int tl_flash_prefill(const void* q, int64_t q_stride, const void* k_cache, const
                      const int32_t* block_tables, int max_blocks, const int32_t* tile_req,
                      const int32_t* tile_tok0, const int32_t* tile_ntok, const int32_t* positions, void* out,
                      int64_t out_stride, float* part_o, float* part_ml, int n_tiles, int n_tokens, int nq, int nkv,
-                     int hd, int block_size, float scale, int window, int tile_waves, int n_splits,
+                     int hd, int block_size, float scale, int window, int sink, int tile_waves, int n_splits,
                      hipStream_t stream) {
   if (n_tiles <= 0) return TL_OK;
   if (tile_waves != 8 && tile_waves != 4) return TL_ERR_ARG;
@@ -1495,7 +1510,7 @@ int tl_flash_prefill(const void* q, int64_t q_stride, const void* k_cache, const
                      stream, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache,          \
                      block_tables, max_blocks, tile_req, tile_tok0, tile_ntok, positions, (bf16_t*)out,           \
                      out_stride, part_o, part_ml, n_tiles, n_tokens, n_splits, nq, nkv, block_size, bs_shift,     \
-                     scale, window)
+                     scale, window, sink)
 #define TL_PREFILL_CASE(HDT)                        \
   case HDT:                                         \
     if (tile_waves == 8) TL_PREFILL_LAUNCH(HDT, 8); \
@@ -1509,7 +1524,7 @@ int tl_flash_prefill(const void* q, int64_t q_stride, const void* k_cache, const
 #undef TL_PREFILL_LAUNCH
 #define TL_COMBINE(B)                                                                                          \
   hipLaunchKernelGGL(flash_combine_kernel<B>, dim3(n_tokens, nq), dim3(TL_WAVE), 0, stream, part_o, part_ml, \
-                     (bf16_t*)out, out_stride, n_tokens, nq, hd, n_splits)
+                     (bf16_t*)out, out_stride, n_tokens, nq, hd, n_splits, sink)
   if (n_splits > 8) TL_COMBINE(16);
   else if (n_splits > 4) TL_COMBINE(8);
   else if (n_splits > 2) TL_COMBINE(4);
@@ -1529,7 +1544,7 @@ static int flash_attention_any(const void* q, int64_t q_stride, const void* k_ca
                                const int32_t* block_tables, int max_blocks, const int32_t* tile_req,
                                const int32_t* tile_tok0, const int32_t* tile_ntok, const int32_t* positions, void* out,
                                int64_t out_stride, float* part_o, float* part_ml, int n_tiles, int n_tokens, int nq,
-                               int nkv, int hd, int block_size, float scale, int window, int n_splits,
+                               int nkv, int hd, int block_size, float scale, int window, int sink, int n_splits,
                                const float* rope_cos, const float* rope_sin, int fuse_store, hipStream_t stream) {
   if (n_tiles <= 0 || n_tokens <= 0) return TL_OK;
   if (nq <= 0 || nkv <= 0 || nq % nkv || nq / nkv > 16 || hd <= 0 || hd % 16 || hd > 128 || block_size <= 0 ||
@@ -1548,7 +1563,7 @@ static int flash_attention_any(const void* q, int64_t q_stride, const void* k_ca
   case HDT:                                                                                                      \
     rc = launch_flash<HDT>((const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache,           \
                            block_tables, max_blocks, tile_req, tile_tok0, tile_ntok, positions, (bf16_t*)out,    \
-                           out_stride, part_o, part_ml, n_tiles, n_tokens, nq, nkv, block_size, scale, window,   \
+                           out_stride, part_o, part_ml, n_tiles, n_tokens, nq, nkv, block_size, scale, window, sink,   \
                            n_splits, fused, stream);                                                             \
     break;
   switch (hd / 16) {
@@ -1559,7 +1574,7 @@ static int flash_attention_any(const void* q, int64_t q_stride, const void* k_ca
   if (rc != TL_OK) return rc;
 #define TL_COMBINE(B)                                                                                          \
   hipLaunchKernelGGL(flash_combine_kernel<B>, dim3(n_tokens, nq), dim3(TL_WAVE), 0, stream, part_o, part_ml, \
-                     (bf16_t*)out, out_stride, n_tokens, nq, hd, n_splits)
+                     (bf16_t*)out, out_stride, n_tokens, nq, hd, n_splits, sink)
   if (n_splits > 8) TL_COMBINE(16);
   else if (n_splits > 4) TL_COMBINE(8);
   else if (n_splits > 2) TL_COMBINE(4);
@@ -1572,11 +1587,11 @@ int tl_flash_attention(const void* q, int64_t q_stride, const void* k_cache, con
                        const int32_t* block_tables, int max_blocks, const int32_t* tile_req,
                        const int32_t* tile_tok0, const int32_t* tile_ntok, const int32_t* positions, void* out,
                        int64_t out_stride, float* part_o, float* part_ml, int n_tiles, int n_tokens, int nq,
-                       int nkv, int hd, int block_size, float scale, int window, int n_splits,
+                       int nkv, int hd, int block_size, float scale, int window, int sink, int n_splits,
                        const float* rope_cos, const float* rope_sin, int fuse_store, hipStream_t stream) {
   return flash_attention_any(q, q_stride, k_cache, v_cache, block_tables, max_blocks, tile_req, tile_tok0, tile_ntok,
                              positions, out, out_stride, part_o, part_ml, n_tiles, n_tokens, nq, nkv, hd, block_size,
-                             scale, window, n_splits, rope_cos, rope_sin, fuse_store, stream);
+                             scale, window, sink, n_splits, rope_cos, rope_sin, fuse_store, stream);
 }
 
 // ------------------------------------------------ the entry point that allocates nothing
@@ -1609,7 +1624,7 @@ int tl_flash_attention_static(const void* q, int64_t q_stride, const void* k_cac
                               const int32_t* block_tables, int max_blocks, const int32_t* tile_req,
                               const int32_t* tile_tok0, const int32_t* tile_ntok, const int32_t* positions,
                               void* out, int64_t out_stride, int n_tiles, int n_tokens, int nq, int nkv, int hd,
-                              int block_size, float scale, int window, int n_splits, const float* rope_cos,
+                              int block_size, float scale, int window, int sink, int n_splits, const float* rope_cos,
                               const float* rope_sin, int fuse_store, hipStream_t stream) {
   if (n_tiles <= 0 || n_tokens <= 0) return TL_OK;
   if (n_splits < 1 || nq <= 0 || hd <= 0) return TL_ERR_ARG;
@@ -1629,7 +1644,7 @@ int tl_flash_attention_static(const void* q, int64_t q_stride, const void* k_cac
   }
   return flash_attention_any(q, q_stride, k_cache, v_cache, block_tables, max_blocks, tile_req, tile_tok0, tile_ntok,
                              positions, out, out_stride, part_o, part_ml, n_tiles, n_tokens, nq, nkv, hd, block_size,
-                             scale, window, n_splits, rope_cos, rope_sin, fuse_store, stream);
+                             scale, window, sink, n_splits, rope_cos, rope_sin, fuse_store, stream);
 }
 
 }  // extern "C"

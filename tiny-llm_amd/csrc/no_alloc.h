@@ -31,7 +31,7 @@ int tl_flash_attention_static(const void* q, int64_t q_stride, const void* k_cac
                               const int32_t* block_tables, int max_blocks, const int32_t* tile_req,
                               const int32_t* tile_tok0, const int32_t* tile_ntok, const int32_t* positions,
                               void* out, int64_t out_stride, int n_tiles, int n_tokens, int nq, int nkv, int hd,
-                              int block_size, float scale, int window, int n_splits, const float* rope_cos,
+                              int block_size, float scale, int window, int sink, int n_splits, const float* rope_cos,
                               const float* rope_sin, int fuse_store, hipStream_t stream);
 
 // The capacity of the static array, in floats.

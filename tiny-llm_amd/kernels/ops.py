@@ -649,7 +649,7 @@ def attention_f32_supported(dtype: torch.dtype, num_heads: int, num_kv_heads: in
 def attention_f32(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                   tiles, positions: torch.Tensor, out: torch.Tensor, num_heads: int, num_kv_heads: int,
                   head_dim: int, scale: float, window: int = 0, n_chunks: int = 1,
-                  scratch: Optional[torch.Tensor] = None) -> torch.Tensor:
+                  scratch: Optional[torch.Tensor] = None, sink: bool = False) -> torch.Tensor:
     """The same function as `paged_attention` in true float32 on the matrix cores.  `tiles` as for
     `flash_attention` (None: row i is the one new token of request i).  n_chunks == 1: one
     workgroup per tile and kv head walks all keys; n_chunks > 1 (at least ceil(longest context /
@@ -696,7 +696,7 @@ def attention_f32(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
         _ptr(q, 16), c_int64(q.stride(0)), _ptr(k_cache, 16), _ptr(v_cache, 16), _ptr(block_tables),
         c_int(block_tables.shape[1]), _ptr(tile_req), _ptr(tile_tok0), _ptr(tile_ntok), _ptr(positions),
         _ptr(out), c_int64(out.stride(0)), _ptr(scratch), c_int(n_tiles), c_int(T), c_int(num_heads),
-        c_int(num_kv_heads), c_int(head_dim), c_int(k_cache.shape[2]), c_float(scale), c_int(window),
+        c_int(num_kv_heads), c_int(head_dim), c_int(k_cache.shape[2]), c_float(scale), c_int(window), c_int(1 if sink else 0),
         c_int(n_chunks), _stream()), "attention_f32")
     return out
 
@@ -710,7 +710,8 @@ def flash_attention_supported(dtype: torch.dtype, num_heads: int, num_kv_heads: 
 def flash_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                     tiles, positions: torch.Tensor, out: torch.Tensor, num_heads: int, num_kv_heads: int,
                     head_dim: int, scale: float, window: int = 0, n_splits: int = 1,
-                    scratch: Optional[torch.Tensor] = None, fused_rope=None, static_scratch: bool = False) -> torch.Tensor:
+                    scratch: Optional[torch.Tensor] = None, fused_rope=None, static_scratch: bool = False,
+                    sink: bool = False) -> torch.Tensor:
     """The same function as `paged_attention` on the matrix cores (bfloat16).  `tiles` =
     (tile_req, tile_tok0, tile_ntok): groups of at most 16 // (heads / kv_heads) consecutive
     tokens of one request; None for a decode step, where row i is the one new token of request i
@@ -781,7 +782,7 @@ def flash_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
             _ptr(q, 16), c_int64(q.stride(0)), _ptr(k_cache, 16), _ptr(v_cache, 16), _ptr(block_tables),
             c_int(block_tables.shape[1]), _ptr(tile_req), _ptr(tile_tok0), _ptr(tile_ntok), _ptr(positions),
             _ptr(out, 8), c_int64(out.stride(0)), c_int(n_tiles), c_int(T), c_int(num_heads), c_int(num_kv_heads),
-            c_int(head_dim), c_int(k_cache.shape[2]), c_float(scale), c_int(window), c_int(n_splits), _ptr(cos),
+            c_int(head_dim), c_int(k_cache.shape[2]), c_float(scale), c_int(window), c_int(1 if sink else 0), c_int(n_splits), _ptr(cos),
             _ptr(sin), c_int(1 if fused_rope is not None else 0), _stream())
         if code == 3:
             _fail(f"split attention over the library's static scratch: {n_splits} splits x {T} tokens x {num_heads} "
@@ -793,7 +794,7 @@ def flash_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         c_int(block_tables.shape[1]), _ptr(tile_req), _ptr(tile_tok0), _ptr(tile_ntok), _ptr(positions),
         _ptr(out, 8), c_int64(out.stride(0)), _ptr(part_o), _ptr(part_ml), c_int(n_tiles), c_int(T),
         c_int(num_heads), c_int(num_kv_heads), c_int(head_dim), c_int(k_cache.shape[2]), c_float(scale),
-        c_int(window), c_int(n_splits), _ptr(cos), _ptr(sin), c_int(1 if fused_rope is not None else 0),
+        c_int(window), c_int(1 if sink else 0), c_int(n_splits), _ptr(cos), _ptr(sin), c_int(1 if fused_rope is not None else 0),
         _stream()), "flash_attention")
     return out
 
@@ -883,7 +884,7 @@ def prefill_tile_waves(num_tokens: int, num_heads: int, num_kv_heads: int) -> in
 def flash_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                   tiles, positions: torch.Tensor, out: torch.Tensor, num_heads: int, num_kv_heads: int,
                   head_dim: int, scale: float, window: int = 0, tile_waves: int = 8, n_splits: int = 1,
-                  scratch: Optional[torch.Tensor] = None) -> torch.Tensor:
+                  scratch: Optional[torch.Tensor] = None, sink: bool = False) -> torch.Tensor:
     """`flash_attention` arranged for prompt portions: `tiles` are groups of at most
     tile_waves * (16 // (heads / kv_heads)) consecutive tokens of one request, and a key or value
     row is staged once per such group.  tile_waves is PREFILL_TILES (8), or 4 for steps with few
@@ -933,7 +934,7 @@ def flash_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
         c_int(block_tables.shape[1]), _ptr(tile_req), _ptr(tile_tok0), _ptr(tile_ntok), _ptr(positions),
         _ptr(out, 8), c_int64(out.stride(0)), _ptr(part_o, 16), _ptr(part_ml), c_int(n_tiles), c_int(T),
         c_int(num_heads), c_int(num_kv_heads),
-        c_int(head_dim), c_int(k_cache.shape[2]), c_float(scale), c_int(window), c_int(tile_waves), c_int(n_splits),
+        c_int(head_dim), c_int(k_cache.shape[2]), c_float(scale), c_int(window), c_int(1 if sink else 0), c_int(tile_waves), c_int(n_splits),
         _stream()), "flash_prefill")
     return out
 

@@ -101,33 +101,31 @@ class Attention(Mixer):
         T, device = q.shape[0], q.device
         group = self.num_heads // self.num_kv_heads
         flash = ops.flash_attention_supported(self.dtype, self.num_heads, self.num_kv_heads, self.head_dim)
-        if sink:
-            # the kernel that takes every size is the one that knows the sink
-            return ops.paged_attention(q, cache.k, cache.v, ctx.block_tables[cache.group], ctx.req_of_token,
-                                       ctx.positions, attn, self.num_heads, self.num_kv_heads, self.head_dim,
-                                       self.scale, self.window, sink=True)
+        # the keys one row walks at most: a window bounds them whatever the context (the kernels begin at the
+        # window's first key tile)
+        span = min(ctx.max_seq_len, self.window + 63) if self.window else ctx.max_seq_len
         if flash and ctx.max_q_len > 1:
             # prompt portions: many query rows share each staged key tile
             waves = ops.prefill_tile_waves(T, self.num_heads, self.num_kv_heads)
             tiles = ctx.attention_tiles(waves * (16 // group))
             # a portion late in a long prompt: few query rows, many keys; the keys are shared out
-            n_splits = ops.prefill_key_splits(T, ctx.max_seq_len, self.num_heads, self.num_kv_heads, waves)
+            n_splits = ops.prefill_key_splits(T, span, self.num_heads, self.num_kv_heads, waves)
             scratch = None
             if n_splits > 1:
                 scratch = ops.scratch("attention_partials", (n_splits * T * self.num_heads * (self.head_dim + 2),),
                                       torch.float32, device)
             ops.flash_prefill(q, cache.k, cache.v, ctx.block_tables[cache.group], tiles, ctx.positions, attn,
                               self.num_heads, self.num_kv_heads, self.head_dim, self.scale, self.window, waves,
-                              n_splits, scratch)
+                              n_splits, scratch, sink=sink)
         elif flash:
             # decoding: one token per request, its keys split over the waves of a workgroup (and over
             # workgroups when the context is long)
             # (no tile arrays when every request brings exactly one token: row i is request i)
             tiles = None if T == ctx.num_requests else ctx.attention_tiles(16 // group)
-            n_splits, scratch = self._splits(ctx, T, device)
+            n_splits, scratch = self._splits(span, T, device)
             ops.flash_attention(q, cache.k, cache.v, ctx.block_tables[cache.group], tiles, ctx.positions, attn,
                                 self.num_heads, self.num_kv_heads, self.head_dim, self.scale, self.window,
-                                n_splits, scratch, fused_rope=fused_rope)
+                                n_splits, scratch, fused_rope=fused_rope, sink=sink)
         elif ops.attention_f32_supported(self.dtype, self.num_heads, self.num_kv_heads, self.head_dim) \
                 and q.stride(0) % 4 == 0:
             # true float32 on the matrix cores; one fixed merge tree, so the same bits whatever the batch
@@ -140,17 +138,17 @@ class Attention(Mixer):
                                       torch.float32, device)
             ops.attention_f32(q, cache.k, cache.v, ctx.block_tables[cache.group], tiles, ctx.positions, attn,
                               self.num_heads, self.num_kv_heads, self.head_dim, self.scale, self.window, n_chunks,
-                              scratch)
+                              scratch, sink=sink)
         else:
             ops.paged_attention(q, cache.k, cache.v, ctx.block_tables[cache.group], ctx.req_of_token,
                                 ctx.positions, attn, self.num_heads, self.num_kv_heads, self.head_dim,
-                                self.scale, self.window)
+                                self.scale, self.window, sink=sink)
         return attn
 
-    def _splits(self, ctx, T: int, device):
-        """How many workgroups share one query tile's keys (`ops.decode_key_splits`), and the scratch
-        for their partial results."""
-        n_splits = ops.decode_key_splits(T, ctx.max_seq_len, self.num_kv_heads, self.head_dim)
+    def _splits(self, span: int, T: int, device):
+        """How many workgroups share one query tile's keys (`ops.decode_key_splits`; `span`: the most keys a
+        row walks), and the scratch for their partial results."""
+        n_splits = ops.decode_key_splits(T, span, self.num_kv_heads, self.head_dim)
         if n_splits == 1:
             return 1, None
         return n_splits, ops.scratch("attention_partials", (n_splits * T * self.num_heads * (self.head_dim + 2),),
