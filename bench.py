@@ -740,7 +740,8 @@ def kernels_by_name(run):
         if m:
             name = e.name[m.end():m.end() + int(m.group(1))]
         else:
-            name = e.name.split("<")[0].split("(")[0].replace("void ", "").strip() or "(unnamed)"
+            plain = e.name.replace("void ", "").replace("(anonymous namespace)::", "")
+            name = plain.split("<")[0].split("(")[0].strip() or "(unnamed)"
         t, n = out.get(name, (0.0, 0))
         out[name] = (t + (e.time_range.end - e.time_range.start), n + 1)
     return {k: {"us": round(t / steps, 1), "launches": round(n / steps, 1)} for k, (t, n) in sorted(out.items(), key=lambda kv: -kv[1][0])}

@@ -528,3 +528,38 @@ def test_table_moe_kernels(dtype):
     s = torch.empty(T, device="cuda")
     ops.row_dot_sigmoid(h.cuda(), sg.cuda(), s)
     assert (s.double().cpu() - torch.sigmoid(h.double() @ sg.double())).abs().max() < 1e-5
+
+
+@pytest.mark.parametrize("T,top,E,N,K", [(70, 3, 5, 72, 40), (33, 1, 3, 300, 64), (200, 2, 2, 16, 104), (64, 2, 9, 260, 32)])
+def test_rows_grouped_by_expert_on_the_matrix_cores(T, top, E, N, K):
+    """Many rows: sorted by expert on the device, tiles of 32 rows of one expert; experts with no row, with one,
+    with more than a tile; column counts that fill no tile; every row against its own expert's weights."""
+    from tiny_llm_amd.kernels import ops
+    g = torch.Generator().manual_seed(T)
+    V = 40
+    h = torch.randn(T, K, generator=g).to(torch.bfloat16)
+    w = (torch.randn(E, N, K, generator=g) / K ** 0.5).to(torch.bfloat16)
+    table = torch.stack([torch.randperm(E, generator=g)[:top] for _ in range(V)]).to(torch.int32)
+    if E > 2:
+        table[table == E - 1] = 0 if top == 1 else table[table == E - 1]      # (top 1: the last expert gets no row)
+    tokens = torch.randint(0, V, (T,), generator=g).to(torch.int32)
+    rows = T * top
+    plan = torch.full((ops.moe_plan_ints(rows, E),), -7, dtype=torch.int32, device="cuda")
+    ops.moe_plan(tokens.cuda(), table.cuda(), plan, E)
+    counts = plan[:E].cpu()
+    want_counts = torch.bincount(table[tokens.long()].reshape(-1).long(), minlength=E)
+    assert torch.equal(counts.long(), want_counts)
+    mt = ops.moe_max_tiles(rows, E)
+    sorted_rows = plan[3 * E + 2 + 3 * mt:3 * E + 2 + 3 * mt + rows].cpu()
+    assert sorted(sorted_rows.tolist()) == list(range(rows))
+    for out_dtype, a, div in ((torch.bfloat16, h, top), (torch.float32, h.repeat_interleave(top, 0), 1)):
+        out = torch.full((rows, N), float("nan"), dtype=out_dtype, device="cuda")
+        ops.grouped_rows_gemm(a.cuda(), div, w.cuda(), plan, out)
+        for r in range(rows):
+            want = w[table[tokens[r // top], r % top]].double() @ h[r // top].double()
+            assert (out[r].double().cpu() - want).abs().max() < (3e-2 if out_dtype == torch.bfloat16 else 1e-4), (r, out_dtype)
+    y, base, sc = torch.randn(rows, N, generator=g), torch.randn(T, N, generator=g), torch.rand(T, generator=g)
+    out = base.clone().cuda()
+    ops.moe_combine(y.cuda().reshape(-1), out, top, 0.5, out, sc.cuda())
+    want = base.double() * sc.double()[:, None] + 0.5 * y.double().reshape(T, top, N).sum(1)
+    assert (out.double().cpu() - want).abs().max() < 1e-5

@@ -105,9 +105,202 @@ __global__ __launch_bounds__(TL_WAVE) void row_dot_sigmoid_kernel(const T* __res
   if (threadIdx.x == 0) out[blockIdx.x] = 1.f / (1.f + expf(-v));
 }
 
+// ------------------------------------------------------------------ many rows: grouped by expert
+// Steps with many rows sort them by expert on the device and multiply tiles of 32 rows of ONE expert on
+// the matrix cores, so that an expert's weights are read once per tile and not once per row.  The plan is
+// a few arrays of int32: counts[E], cursor[E], offsets[E + 1], n_tiles, then per tile its expert, its first
+// place in `sorted` and its number of rows, then sorted[rows] (the row indices t * top + j by expert; the
+// order inside an expert is whatever the atomics give: a row's result does not depend on its place).
+constexpr int kTileRows = 32;
+
+__global__ void moe_count_kernel(const int32_t* __restrict__ tokens, const int32_t* __restrict__ table,
+                                 int32_t* __restrict__ counts, int rows, int top, int experts, int vocab) {
+  const int i = blockIdx.x * kThreads + threadIdx.x;
+  if (i >= rows) return;
+  atomicAdd(&counts[expert_of(tokens, table, i / top, i % top, top, vocab, experts)], 1);
+}
+
+// One workgroup: offsets of the experts' runs in `sorted`, and the list of tiles.
+__global__ __launch_bounds__(kThreads) void moe_plan_kernel(const int32_t* __restrict__ counts,
+                                                            int32_t* __restrict__ cursor, int32_t* __restrict__ offsets,
+                                                            int32_t* __restrict__ n_tiles,
+                                                            int32_t* __restrict__ tile_expert,
+                                                            int32_t* __restrict__ tile_start,
+                                                            int32_t* __restrict__ tile_rows, int experts, int max_tiles) {
+  __shared__ int32_t first_tile[1025];
+  if (threadIdx.x == 0) {
+    int at = 0, nt = 0;
+    for (int e = 0; e < experts; ++e) {
+      offsets[e] = at;
+      first_tile[e] = nt;
+      at += counts[e];
+      nt += (counts[e] + kTileRows - 1) / kTileRows;
+    }
+    offsets[experts] = at;
+    first_tile[experts] = nt;
+    n_tiles[0] = min(nt, max_tiles);
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < experts; e += kThreads) {
+    cursor[e] = 0;
+    const int c = counts[e];
+    for (int i = 0, t = first_tile[e]; i * kTileRows < c && t < max_tiles; ++i, ++t) {
+      tile_expert[t] = e;
+      tile_start[t] = offsets[e] + i * kTileRows;
+      tile_rows[t] = min(kTileRows, c - i * kTileRows);
+    }
+  }
+}
+
+__global__ void moe_scatter_kernel(const int32_t* __restrict__ tokens, const int32_t* __restrict__ table,
+                                   const int32_t* __restrict__ offsets, int32_t* __restrict__ cursor,
+                                   int32_t* __restrict__ sorted, int rows, int top, int experts, int vocab) {
+  const int i = blockIdx.x * kThreads + threadIdx.x;
+  if (i >= rows) return;
+  const int e = expert_of(tokens, table, i / top, i % top, top, vocab, experts);
+  sorted[offsets[e] + atomicAdd(&cursor[e], 1)] = i;
+}
+
+// out[row, n] = sum_k a[row / a_div, k] * w[expert of row][n, k] for the rows of one tile; bfloat16 operands
+// straight from memory into v_mfma_f32_16x16x32_bf16 (weights as the first operand, so that a lane holds four
+// neighbouring columns of one row), float32 sums.  A workgroup of four waves owns 32 rows x 256 columns, a wave
+// 32 x 64: six operand loads per eight matrix instructions.
+template <typename TO>
+__global__ __launch_bounds__(kThreads) void grouped_rows_gemm_bf16_kernel(
+    const bf16_t* __restrict__ a, int64_t a_stride, int a_div, const bf16_t* __restrict__ w, TO* __restrict__ out,
+    const int32_t* __restrict__ n_tiles, const int32_t* __restrict__ tile_expert, const int32_t* __restrict__ tile_start,
+    const int32_t* __restrict__ tile_rows, const int32_t* __restrict__ sorted, int N, int K) {
+  const int tile = blockIdx.x;
+  if (tile >= n_tiles[0]) return;
+  const int e = tile_expert[tile], start = tile_start[tile], nrows = tile_rows[tile];
+  const int wave = threadIdx.x / TL_WAVE, lane = threadIdx.x % TL_WAVE, r16 = lane % 16, kq = lane / 16;
+  const int col0 = blockIdx.y * 256 + wave * 64;
+  if (col0 >= N) return;
+  int src[2];
+  const bf16_t* ap[2];
+#pragma unroll
+  for (int rb = 0; rb < 2; ++rb) {
+    src[rb] = sorted[start + min(rb * 16 + r16, nrows - 1)];
+    ap[rb] = a + (int64_t)(src[rb] / a_div) * a_stride + kq * 8;
+  }
+  const bf16_t* wp[4];
+#pragma unroll
+  for (int cb = 0; cb < 4; ++cb) wp[cb] = w + ((int64_t)e * N + min(col0 + cb * 16 + r16, N - 1)) * K + kq * 8;
+  f32x4 acc[2][4];
+#pragma unroll
+  for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+    for (int cb = 0; cb < 4; ++cb) acc[rb][cb] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const bool second = nrows > 16;
+  for (int k0 = 0; k0 < K; k0 += 32) {
+    const bool in = k0 + kq * 8 < K;                // K is a multiple of 8
+    bf16x8 af[2], wf[4];
+    const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb) af[rb] = in ? *(const bf16x8*)(ap[rb] + k0) : zero;
+#pragma unroll
+    for (int cb = 0; cb < 4; ++cb) wf[cb] = in ? *(const bf16x8*)(wp[cb] + k0) : zero;
+#pragma unroll
+    for (int cb = 0; cb < 4; ++cb) {
+      acc[0][cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[cb], af[0], acc[0][cb], 0, 0, 0);
+      if (second) acc[1][cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[cb], af[1], acc[1][cb], 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int rb = 0; rb < 2; ++rb) {
+    if (rb * 16 + r16 >= nrows) continue;
+    TO* orow = out + (int64_t)src[rb] * N;
+#pragma unroll
+    for (int cb = 0; cb < 4; ++cb)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int c = col0 + cb * 16 + kq * 4 + i;
+        if (c < N) orow[c] = from_f32<TO>(acc[rb][cb][i]);
+      }
+  }
+}
+
+// out[t, c] = base[t, c] * base_scale[t] + coef * sum_j y[t * top + j, c]   (the experts in the table's order)
+__global__ void moe_combine_kernel(const float* __restrict__ y, const float* __restrict__ base,
+                                   const float* __restrict__ base_scale, float* __restrict__ out, int64_t total, int N,
+                                   int top, float coef) {
+  const int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (i >= total) return;
+  const int64_t t = i / N;
+  const int c = (int)(i - t * N);
+  float acc = 0.f;
+  for (int j = 0; j < top; ++j) acc += y[(t * top + j) * N + c];
+  const float b = base ? base[i] * (base_scale ? base_scale[t] : 1.f) : 0.f;
+  out[i] = fmaf(coef, acc, b);
+}
+
 }  // namespace
 
 extern "C" {
+
+int tl_moe_tile_rows(void) { return kTileRows; }
+
+// plan: int32 [2 * experts + (experts + 1) + 1 + 3 * max_tiles + n_tokens * top], counts and cursor zeroed by the
+// caller; max_tiles >= ceil(n_tokens * top / 32) + experts.
+int tl_moe_plan(const int32_t* tokens, const int32_t* table, int32_t* plan, int n_tokens, int top, int experts, int vocab,
+                int max_tiles, hipStream_t stream) {
+  if (n_tokens <= 0) return TL_OK;
+  const int64_t rows = (int64_t)n_tokens * top;
+  if (top <= 0 || experts <= 0 || experts > 1024 || vocab <= 0 || rows > 0x7fffffff || !tokens || !table || !plan ||
+      max_tiles < (rows + kTileRows - 1) / kTileRows + experts)
+    return TL_ERR_ARG;
+  int32_t* counts = plan;
+  int32_t* cursor = counts + experts;
+  int32_t* offsets = cursor + experts;
+  int32_t* n_tiles = offsets + experts + 1;
+  int32_t* tile_expert = n_tiles + 1;
+  int32_t* tile_start = tile_expert + max_tiles;
+  int32_t* tile_rows = tile_start + max_tiles;
+  int32_t* sorted = tile_rows + max_tiles;
+  const unsigned blocks = (unsigned)ceil_div64(rows, kThreads);
+  hipLaunchKernelGGL(moe_count_kernel, dim3(blocks), dim3(kThreads), 0, stream, tokens, table, counts, (int)rows, top,
+                     experts, vocab);
+  hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(kThreads), 0, stream, counts, cursor, offsets, n_tiles, tile_expert,
+                     tile_start, tile_rows, experts, max_tiles);
+  hipLaunchKernelGGL(moe_scatter_kernel, dim3(blocks), dim3(kThreads), 0, stream, tokens, table, offsets, cursor, sorted,
+                     (int)rows, top, experts, vocab);
+  return tl_launch_status();
+}
+
+// a: bfloat16 rows (row r of the plan reads a[r / a_div]); w: bfloat16 [experts, N, K]; out: [rows, N] bfloat16
+// (out_dtype 1) or float32 (0), written at the rows' own places.
+int tl_grouped_rows_gemm(const void* a, int64_t a_stride, int a_div, const void* w, void* out, const int32_t* plan,
+                         int n_rows, int experts, int max_tiles, int N, int K, int out_dtype, hipStream_t stream) {
+  if (n_rows <= 0) return TL_OK;
+  if (a_div <= 0 || experts <= 0 || N <= 0 || K <= 0 || K % 8 || a_stride % 8 || a_stride < K || !a || !w || !out || !plan ||
+      max_tiles <= 0 || (N + 255) / 256 > 65535)
+    return TL_ERR_ARG;
+  const int32_t* n_tiles = plan + 3 * experts + 1;
+  const int32_t* tile_expert = n_tiles + 1;
+  const int32_t* tile_start = tile_expert + max_tiles;
+  const int32_t* tile_rows = tile_start + max_tiles;
+  const int32_t* sorted = tile_rows + max_tiles;
+  dim3 g(max_tiles, (N + 255) / 256), b(kThreads);
+  if (out_dtype == 1)
+    hipLaunchKernelGGL(grouped_rows_gemm_bf16_kernel<bf16_t>, g, b, 0, stream, (const bf16_t*)a, a_stride, a_div,
+                       (const bf16_t*)w, (bf16_t*)out, n_tiles, tile_expert, tile_start, tile_rows, sorted, N, K);
+  else if (out_dtype == 0)
+    hipLaunchKernelGGL(grouped_rows_gemm_bf16_kernel<float>, g, b, 0, stream, (const bf16_t*)a, a_stride, a_div,
+                       (const bf16_t*)w, (float*)out, n_tiles, tile_expert, tile_start, tile_rows, sorted, N, K);
+  else
+    return TL_ERR_ARG;
+  return tl_launch_status();
+}
+
+int tl_moe_combine(const float* y, const float* base, const float* base_scale, float* out, int n_tokens, int N, int top,
+                   float coef, hipStream_t stream) {
+  if (n_tokens <= 0) return TL_OK;
+  if (N <= 0 || top <= 0 || !y || !out) return TL_ERR_ARG;
+  const int64_t total = (int64_t)n_tokens * N;
+  hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)ceil_div64(total, kThreads)), dim3(kThreads), 0, stream, y, base,
+                     base_scale, out, total, N, top, coef);
+  return tl_launch_status();
+}
 
 // a: [n_tokens, K] (row stride a_stride); w: [experts, N, K]; table: int32 [vocab, top]; out: [n_tokens * top, N].
 int tl_table_moe_up(const void* a, int64_t a_stride, const void* w, const int32_t* tokens, const int32_t* table, void* out,

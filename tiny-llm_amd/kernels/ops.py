@@ -1794,6 +1794,70 @@ def table_moe_down(z: torch.Tensor, w: torch.Tensor, tokens: torch.Tensor, table
     return out
 
 
+MOE_TILE_ROWS = 32          # rows of one expert a tile of the grouped product holds (csrc/moe.hip)
+
+
+def moe_max_tiles(rows: int, experts: int) -> int:
+    return -(-rows // MOE_TILE_ROWS) + experts
+
+
+def moe_plan_ints(rows: int, experts: int) -> int:
+    """int32 elements of the plan `moe_plan` fills for `rows` (= tokens * top) rows."""
+    return 3 * experts + 2 + 3 * moe_max_tiles(rows, experts) + rows
+
+
+def moe_plan(tokens: torch.Tensor, table: torch.Tensor, plan: torch.Tensor, experts: int) -> torch.Tensor:
+    """Sorts the step's rows (token t, its j-th expert: row t * top + j) by expert on the device and lists
+    tiles of at most 32 rows of one expert each; `plan` is int32 scratch of `moe_plan_ints` elements."""
+    _dev(tokens, table, plan)
+    _i32(tokens, table, plan)
+    V, top = table.shape
+    T = tokens.numel()
+    _need(plan.numel() >= moe_plan_ints(T * top, experts), "moe_plan: the plan is too short")
+    _need(0 < experts <= 1024, "moe_plan: 1 to 1024 experts")
+    plan[:2 * experts].zero_()          # counts and cursors (a fill kernel: fine inside a captured step)
+    _check(_lib().tl_moe_plan(_ptr(tokens), _ptr(table), _ptr(plan), c_int(T), c_int(top), c_int(experts), c_int(V),
+                              c_int(moe_max_tiles(T * top, experts)), _stream()), "moe_plan")
+    return plan
+
+
+def grouped_rows_gemm(a: torch.Tensor, a_div: int, w: torch.Tensor, plan: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[r] = w[expert of row r] @ a[r // a_div] for every row r of the plan, on the matrix cores (bfloat16
+    operands, float32 sums); a [*, K], w [E, N, K] bfloat16, out contiguous [rows, N] bfloat16 or float32."""
+    _dev(a, w, plan, out)
+    _rows_2d(a, "grouped_rows_gemm input")
+    E, N, K = w.shape
+    rows = out.shape[0]
+    _need(a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and w.is_contiguous() and a.shape[1] == K,
+          "grouped_rows_gemm: a [*, K] and contiguous w [E, N, K] are bfloat16")
+    _need(K % 8 == 0 and a.stride(0) % 8 == 0, "grouped_rows_gemm: inner size and row stride are multiples of 8")
+    _need(out.is_contiguous() and out.shape[1] == N and a.shape[0] * a_div >= rows,
+          "grouped_rows_gemm: out is contiguous [rows, N], a holds rows / a_div rows")
+    _i32(plan)
+    _need(plan.numel() >= moe_plan_ints(rows, E), "grouped_rows_gemm: the plan is too short")
+    _check(_lib().tl_grouped_rows_gemm(_ptr(a, 16), c_int64(a.stride(0)), c_int(a_div), _ptr(w, 16), _ptr(out),
+                                       _ptr(plan), c_int(rows), c_int(E), c_int(moe_max_tiles(rows, E)), c_int(N),
+                                       c_int(K), c_int(_dt(out)), _stream()), "grouped_rows_gemm")
+    return out
+
+
+def moe_combine(y: torch.Tensor, out: torch.Tensor, top: int, coef: float, base: Optional[torch.Tensor] = None,
+                base_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[t] = base[t] * base_scale[t] + coef * sum_j y[t * top + j]; all float32, out may be base."""
+    _dev(y, out, base, base_scale)
+    T, N = out.shape
+    _need(out.dtype == torch.float32 and out.is_contiguous(), "moe_combine: out is contiguous float32 [T, N]")
+    _f32_vec(y, T * top * N, "moe_combine input")
+    if base is not None:
+        _need(base.dtype == torch.float32 and base.is_contiguous() and base.shape == out.shape,
+              "moe_combine: base is contiguous float32 [T, N]")
+    if base_scale is not None:
+        _f32_vec(base_scale, T, "moe_combine base_scale")
+    _check(_lib().tl_moe_combine(_ptr(y), _ptr(base), _ptr(base_scale), _ptr(out), c_int(T), c_int(N), c_int(top),
+                                 c_float(coef), _stream()), "moe_combine")
+    return out
+
+
 def row_dot_sigmoid(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     """out[t] = sigmoid(a[t] . w); a [T, K] and w [K] of one type, out float32 [T]."""
     _dev(a, w, out)

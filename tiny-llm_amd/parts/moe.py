@@ -20,6 +20,7 @@ from .mlp import ClampedGLU
 
 class TableMoE(FeedForward):
     graph_safe = True
+    GROUPED_ROWS = 64       # from this many rows (tokens * top) on, a bfloat16 step groups its rows by expert
 
     def __init__(self, prefix, dtype, device, *, hidden_size: int, vocab_size: int, num_experts: int, top: int,
                  intermediate_size: int, limit: float, alpha: float = 1.702, shift: float = 1.0,
@@ -79,12 +80,24 @@ class TableMoE(FeedForward):
             base = self.shared.forward(h, ctx, None)
             if self.shared_gate:
                 scale = ops.row_dot_sigmoid(h, self.w_sg, ops.scratch("moe_shared_gate", (T,), torch.float32, dev))
-        gu = ops.scratch("moe_gate_up", (T * self.top, 2 * F), self.dtype, dev)
-        ops.table_moe_up(h, self.w_gate_up, tokens, self.table, gu)
-        z = ops.scratch("moe_gated", (T * self.top, F), self.dtype, dev)
-        ops.clamped_glu(gu, z, self.limit, self.alpha, self.shift)
+        rows = T * self.top
+        gu = ops.scratch("moe_gate_up", (rows, 2 * F), self.dtype, dev)
+        z = ops.scratch("moe_gated", (rows, F), self.dtype, dev)
         out = base if base is not None else ops.scratch("sublayer_out", (T, self.hidden_size), torch.float32, dev)
-        ops.table_moe_down(z, self.w_down, tokens, self.table, out, 1.0 / self.top, base, scale)
+        if self.dtype == torch.bfloat16 and rows >= self.GROUPED_ROWS:
+            # many rows: sorted by expert on the device, tiles of one expert's rows on the matrix cores
+            plan = ops.scratch("moe_plan", (ops.moe_plan_ints(rows, self.num_experts),), torch.int32, dev)
+            ops.moe_plan(tokens, self.table, plan, self.num_experts)
+            ops.grouped_rows_gemm(h, self.top, self.w_gate_up, plan, gu)
+            ops.clamped_glu(gu, z, self.limit, self.alpha, self.shift)
+            y = ops.scratch("moe_rows_out", (rows, self.hidden_size), torch.float32, dev)
+            ops.grouped_rows_gemm(z, 1, self.w_down, plan, y)
+            ops.moe_combine(y, out, self.top, 1.0 / self.top, base, scale)
+        else:
+            # few rows (decoding) and float32: each row against its own expert's weights
+            ops.table_moe_up(h, self.w_gate_up, tokens, self.table, gu)
+            ops.clamped_glu(gu, z, self.limit, self.alpha, self.shift)
+            ops.table_moe_down(z, self.w_down, tokens, self.table, out, 1.0 / self.top, base, scale)
         if residual is None:
             return out
         return add_to_residual(residual, out)
