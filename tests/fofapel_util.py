@@ -46,7 +46,7 @@ def model(width, vocab, layers, alpha, eps=1e-5):
 
 # experts first; windows, head shapes and rotated dims that differ from layer to layer (three cache groups);
 # part of the head rotated, all of it, none of it; one, some and all query heads a kv head; a time mix whose heads
-# are no multiple of the 16-channel slices (24), wider than the attention's (80) and of a single head; ranks that
+# are no power of two of 4-channel slices (24), wider than the attention's (80) and of a single head; ranks that
 # are no multiple of 8; one, two and three experts a token, with a gated shared expert, one without gate, none;
 # a layer without feed-forward
 MIX_A = model(64, 301, [

@@ -53,7 +53,7 @@ def test_cache_groups_and_state_rows():
     assert [caches[(i, "mixer")].window for i in range(4)] == [24, 7, 1000, 33]
     assert all(c.kind == "window" and [t.name for t in c.tensors] == ["k", "v"] for c in caches.values())
     states = dec.state_specs()
-    # S in slices of 16 key channels (24 -> 32, 80 -> 128) plus the last token's input
+    # S in a power of two of slices of 4 key channels (24 -> 32, 80 -> 128) plus the last token's input
     assert states[(0, "mixer")].shape == (2 * 32 * 24 + 64,)
     assert states[(1, "mixer")].shape == (1 * 128 * 80 + 64,)
     assert states[(2, "mixer")].shape == (3 * 16 * 16 + 64,)

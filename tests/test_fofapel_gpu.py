@@ -400,7 +400,7 @@ def test_qk_prepare(dtype, pairing, rot):
 def test_time_mix_state_over_slots_and_tiny_portions(H, D):
     """The shift and the recurrence kernels alone: three requests of unequal length in slots out of order,
     fed in portions of 1 to 7 tokens, against the plain recurrence over each whole sequence; heads that are
-    no multiple of the kernel's 16-channel slices, narrower, and as wide as it takes."""
+    no power of two of the kernel's 4-channel slices, narrow, and as wide as it takes."""
     from tiny_llm_amd.kernels import ops
     g = torch.Generator().manual_seed(9)
     W, S = 40, H * D
@@ -562,4 +562,44 @@ def test_rows_grouped_by_expert_on_the_matrix_cores(T, top, E, N, K):
     out = base.clone().cuda()
     ops.moe_combine(y.cuda().reshape(-1), out, top, 0.5, out, sc.cuda())
     want = base.double() * sc.double()[:, None] + 0.5 * y.double().reshape(T, top, N).sum(1)
+    assert (out.double().cpu() - want).abs().max() < 1e-5
+
+
+@pytest.mark.parametrize("T,top,E,N,K", [(600, 2, 3, 72, 40), (300, 1, 4, 264, 64), (400, 3, 3, 512, 104)])
+def test_runs_of_an_experts_rows_through_the_tiled_product(T, top, E, N, K):
+    """Very many rows: every expert's rows copied side by side into runs of 256, the tiled product with a weight
+    matrix per run (runs without rows skipped), and the sum of a token's rows looked up where they went."""
+    from tiny_llm_amd.kernels import ops
+    g = torch.Generator().manual_seed(T)
+    V, R = 40, ops.MOE_RUN_ROWS
+    h = torch.randn(T, K, generator=g).to(torch.bfloat16)
+    w = (torch.randn(E, N, K, generator=g) / K ** 0.5).to(torch.bfloat16)
+    table = torch.stack([torch.randperm(E, generator=g)[:top] for _ in range(V)]).to(torch.int32)
+    if top == 1:
+        table[table == E - 1] = 0                 # an expert without rows
+    tokens = torch.randint(0, V, (T,), generator=g).to(torch.int32)
+    rows = T * top
+    cap = ops.moe_max_tiles(rows, E, R) * R
+    plan = torch.full((ops.moe_plan_ints(rows, E, R),), -7, dtype=torch.int32, device="cuda")
+    ops.moe_plan(tokens.cuda(), table.cuda(), plan, E, R)
+    runs = ops.moe_tile_experts(plan, rows, E, R)
+    hp = torch.full((cap, K), float("nan"), dtype=torch.bfloat16, device="cuda")
+    pos = torch.full((rows,), -1, dtype=torch.int32, device="cuda")
+    ops.moe_gather(h.cuda(), top, plan, rows, E, R, hp, pos)
+    where = pos.cpu().long()
+    assert len(set(where.tolist())) == rows and int(where.min()) >= 0 and int(where.max()) < cap
+    for out_dtype in (torch.bfloat16, torch.float32):
+        out = torch.full((cap, N), float("nan"), dtype=out_dtype, device="cuda")
+        ops.linear_grouped(hp, w.cuda(), runs, out)
+        got = out.double().cpu()[where]
+        for r in range(0, rows, 7):
+            e = int(table[tokens[r // top], r % top])
+            assert int(runs[where[r] // R]) == e
+            want = w[e].double() @ h[r // top].double()
+            assert (got[r] - want).abs().max() < (3e-2 if out_dtype == torch.bfloat16 else 1e-4), (r, out_dtype)
+    y = torch.randn(cap, N, generator=g)
+    base, sc = torch.randn(T, N, generator=g), torch.rand(T, generator=g)
+    out = base.clone().cuda()
+    ops.moe_combine_at(y.cuda(), pos, out, top, 0.5, out, sc.cuda())
+    want = base.double() * sc.double()[:, None] + 0.5 * y.double()[where].reshape(T, top, N).sum(1)
     assert (out.double().cpu() - want).abs().max() < 1e-5

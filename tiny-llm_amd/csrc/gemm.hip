@@ -469,6 +469,12 @@ struct TileNorm {
   const float* in_sumsq = nullptr;
   int in_parts = 0, in_width = 0;
   float in_eps = 0.f;
+  // Rows in groups with weights of their own: every aligned run of `group_rows` rows (a multiple of every tile
+  // height) multiplies the weight matrix tile_group[run] * group_stride elements behind `w`; a run whose entry is
+  // negative holds no row and is skipped.
+  int group_rows = 0;
+  const int32_t* tile_group = nullptr;
+  int64_t group_stride = 0;
   TileNorm() = default;
   TileNorm(const float* rs) : row_scale(rs) {}
 };
@@ -512,6 +518,11 @@ __global__ __launch_bounds__(WM * WN * TL_WAVE) void gemm_bf16_kernel(const bf16
   const int kbase = split * k_per_split;
   const int kend = k_per_split > 0 ? min(K, kbase + k_per_split) : K;
   if (k_per_split > 0) out += (int64_t)split * M * ldo;
+  if (nm.tile_group) {      // uniform: this tile's rows belong to one group, with weights of its own
+    const int group = nm.tile_group[m0 / nm.group_rows];
+    if (group < 0) return;
+    w += (int64_t)group * nm.group_stride;
+  }
 
   f32x16 acc[MI][NJ];
 #pragma unroll
@@ -1961,6 +1972,30 @@ int tl_linear_handoff(const void* a, const void* w, void* out, const float* resi
     p.in_eps = in_eps;
   }
   const int rc = launch_skinny_out<PRO_NONE>(p, out_dtype, swiglu, stream);
+  if (rc != TL_OK) return rc;
+  return tl_launch_status();
+}
+
+// out = a @ w[g]^T by runs of rows: a bfloat16 [M, K] whose aligned runs of `group_rows` rows (256: a multiple of
+// every tile height; M a multiple of it) each belong to one group g = tile_group[run] (negative: the run holds no
+// row and nothing is computed or written for it); w bfloat16 [groups, N, K]; out [M, N] bfloat16 or float32.
+int tl_linear_grouped(const void* a, const void* w, void* out, const int32_t* tile_group, int group_rows, int M, int N,
+                      int K, int64_t lda, int64_t ldo, int out_dtype, hipStream_t stream) {
+  if (M <= 0) return TL_OK;
+  if (N <= 0 || K <= 0 || K % 8 || lda % 8 || lda < K || ldo < N || (out_dtype != 0 && out_dtype != 1) || !tile_group ||
+      group_rows != 256 || M % group_rows || !a || !w || !out)
+    return TL_ERR_ARG;
+  TileNorm nm;
+  nm.tile_group = tile_group;
+  nm.group_rows = group_rows;
+  nm.group_stride = (int64_t)N * K;
+  int rc;
+  if (out_dtype == 0)
+    rc = launch_gemm_bf16_any<float, false>((const bf16_t*)a, (const bf16_t*)w, (float*)out, nullptr, nm, M, N, K, lda,
+                                            ldo, 0, 0, stream);
+  else
+    rc = launch_gemm_bf16_any<bf16_t, false>((const bf16_t*)a, (const bf16_t*)w, (bf16_t*)out, nullptr, nm, M, N, K, lda,
+                                             ldo, 0, 0, stream);
   if (rc != TL_OK) return rc;
   return tl_launch_status();
 }

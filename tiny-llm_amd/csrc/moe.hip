@@ -126,7 +126,9 @@ __global__ __launch_bounds__(kThreads) void moe_plan_kernel(const int32_t* __res
                                                             int32_t* __restrict__ n_tiles,
                                                             int32_t* __restrict__ tile_expert,
                                                             int32_t* __restrict__ tile_start,
-                                                            int32_t* __restrict__ tile_rows, int experts, int max_tiles) {
+                                                            int32_t* __restrict__ tile_rows, int experts, int max_tiles,
+                                                            int rows_a_tile) {
+  const int kTileRows = rows_a_tile;
   __shared__ int32_t first_tile[1025];
   if (threadIdx.x == 0) {
     int at = 0, nt = 0;
@@ -150,6 +152,46 @@ __global__ __launch_bounds__(kThreads) void moe_plan_kernel(const int32_t* __res
       tile_rows[t] = min(kTileRows, c - i * kTileRows);
     }
   }
+  // tiles behind the last one hold no row
+  for (int t = first_tile[experts] + threadIdx.x; t < max_tiles; t += kThreads) {
+    tile_expert[t] = -1;
+    tile_start[t] = 0;
+    tile_rows[t] = 0;
+  }
+}
+
+// The rows of every tile copied side by side: dst[tile * rows_a_tile + i] = a[sorted row / a_div], and where each
+// row went (row_pos[row] = tile * rows_a_tile + i).  One workgroup a (tile, run of 8 rows).
+__global__ __launch_bounds__(kThreads) void moe_gather_kernel(const bf16_t* __restrict__ a, int64_t a_stride, int a_div,
+                                                              bf16_t* __restrict__ dst, int32_t* __restrict__ row_pos,
+                                                              const int32_t* __restrict__ tile_start,
+                                                              const int32_t* __restrict__ tile_rows,
+                                                              const int32_t* __restrict__ sorted, int K,
+                                                              int rows_a_tile) {
+  const int tile = blockIdx.x, n = tile_rows[tile];
+  for (int i = blockIdx.y * 8; i < min(n, blockIdx.y * 8 + 8); ++i) {
+    const int src = sorted[tile_start[tile] + i];
+    const int64_t at = (int64_t)tile * rows_a_tile + i;
+    if (row_pos && threadIdx.x == 0) row_pos[src] = (int32_t)at;
+    if (a) {
+      const bf16_t* from = a + (int64_t)(src / a_div) * a_stride;
+      for (int k = threadIdx.x * 8; k < K; k += kThreads * 8) *(bf16x8*)(dst + at * K + k) = *(const bf16x8*)(from + k);
+    }
+  }
+}
+
+// out[t, c] = base[t, c] * base_scale[t] + coef * sum_j y[row_pos[t * top + j], c]
+__global__ void moe_combine_at_kernel(const float* __restrict__ y, const int32_t* __restrict__ row_pos,
+                                      const float* __restrict__ base, const float* __restrict__ base_scale,
+                                      float* __restrict__ out, int64_t total, int N, int top, float coef) {
+  const int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (i >= total) return;
+  const int64_t t = i / N;
+  const int c = (int)(i - t * N);
+  float acc = 0.f;
+  for (int j = 0; j < top; ++j) acc += y[(int64_t)row_pos[t * top + j] * N + c];
+  const float b = base ? base[i] * (base_scale ? base_scale[t] : 1.f) : 0.f;
+  out[i] = fmaf(coef, acc, b);
 }
 
 __global__ void moe_scatter_kernel(const int32_t* __restrict__ tokens, const int32_t* __restrict__ table,
@@ -243,11 +285,11 @@ int tl_moe_tile_rows(void) { return kTileRows; }
 // plan: int32 [2 * experts + (experts + 1) + 1 + 3 * max_tiles + n_tokens * top], counts and cursor zeroed by the
 // caller; max_tiles >= ceil(n_tokens * top / 32) + experts.
 int tl_moe_plan(const int32_t* tokens, const int32_t* table, int32_t* plan, int n_tokens, int top, int experts, int vocab,
-                int max_tiles, hipStream_t stream) {
+                int max_tiles, int rows_a_tile, hipStream_t stream) {
   if (n_tokens <= 0) return TL_OK;
   const int64_t rows = (int64_t)n_tokens * top;
   if (top <= 0 || experts <= 0 || experts > 1024 || vocab <= 0 || rows > 0x7fffffff || !tokens || !table || !plan ||
-      max_tiles < (rows + kTileRows - 1) / kTileRows + experts)
+      rows_a_tile <= 0 || max_tiles < (rows + rows_a_tile - 1) / rows_a_tile + experts)
     return TL_ERR_ARG;
   int32_t* counts = plan;
   int32_t* cursor = counts + experts;
@@ -261,7 +303,7 @@ int tl_moe_plan(const int32_t* tokens, const int32_t* table, int32_t* plan, int 
   hipLaunchKernelGGL(moe_count_kernel, dim3(blocks), dim3(kThreads), 0, stream, tokens, table, counts, (int)rows, top,
                      experts, vocab);
   hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(kThreads), 0, stream, counts, cursor, offsets, n_tiles, tile_expert,
-                     tile_start, tile_rows, experts, max_tiles);
+                     tile_start, tile_rows, experts, max_tiles, rows_a_tile);
   hipLaunchKernelGGL(moe_scatter_kernel, dim3(blocks), dim3(kThreads), 0, stream, tokens, table, offsets, cursor, sorted,
                      (int)rows, top, experts, vocab);
   return tl_launch_status();
@@ -289,6 +331,34 @@ int tl_grouped_rows_gemm(const void* a, int64_t a_stride, int a_div, const void*
                        (const bf16_t*)w, (float*)out, n_tiles, tile_expert, tile_start, tile_rows, sorted, N, K);
   else
     return TL_ERR_ARG;
+  return tl_launch_status();
+}
+
+// The plan's rows (tiles of rows_a_tile rows) copied side by side into dst [max_tiles * rows_a_tile, K] (a null: no
+// copy), and row_pos[row] = where it went (null: not wanted).
+int tl_moe_gather(const void* a, int64_t a_stride, int a_div, void* dst, int32_t* row_pos, const int32_t* plan,
+                  int experts, int max_tiles, int rows_a_tile, int K, hipStream_t stream) {
+  if (max_tiles <= 0) return TL_OK;
+  if (a_div <= 0 || experts <= 0 || rows_a_tile <= 0 || K <= 0 || K % 8 || (a && (a_stride % 8 || !dst)) || !plan ||
+      max_tiles > 0x7fffff00 / rows_a_tile)
+    return TL_ERR_ARG;
+  const int32_t* tile_start = plan + 3 * experts + 2 + max_tiles;
+  const int32_t* tile_rows = tile_start + max_tiles;
+  const int32_t* sorted = tile_rows + max_tiles;
+  hipLaunchKernelGGL(moe_gather_kernel, dim3(max_tiles, (rows_a_tile + 7) / 8), dim3(kThreads), 0, stream,
+                     (const bf16_t*)a, a_stride, a_div, (bf16_t*)dst, row_pos, tile_start, tile_rows, sorted, K,
+                     rows_a_tile);
+  return tl_launch_status();
+}
+
+// As tl_moe_combine with the rows of y looked up in row_pos.
+int tl_moe_combine_at(const float* y, const int32_t* row_pos, const float* base, const float* base_scale, float* out,
+                      int n_tokens, int N, int top, float coef, hipStream_t stream) {
+  if (n_tokens <= 0) return TL_OK;
+  if (N <= 0 || top <= 0 || !y || !out || !row_pos) return TL_ERR_ARG;
+  const int64_t total = (int64_t)n_tokens * N;
+  hipLaunchKernelGGL(moe_combine_at_kernel, dim3((unsigned)ceil_div64(total, kThreads)), dim3(kThreads), 0, stream, y,
+                     row_pos, base, base_scale, out, total, N, top, coef);
   return tl_launch_status();
 }
 

@@ -48,25 +48,47 @@ __global__ __launch_bounds__(kThreads) void shift_save_kernel(const T* __restric
 }
 
 // The recurrence.  A workgroup owns EC value columns of one (request, head) and walks the request's
-// tokens of this step in order.  The key channels are cut into P slices of 16 (P a power of two, 16 P >= dim);
-// thread (e, p) keeps S[16 p .. 16 p + 15, e] in registers, and the P lanes of a column are neighbours, so the sum
-// over the channels ends with log2 P lane exchanges.  The order of additions is the same whatever the step holds.
-// r, k and the decays of 16 tokens at a time are staged in LDS.  In memory S lies as [head][s][e][p]
-// (s the index within a slice): a wave's accesses to the state are contiguous.
-constexpr int kSlice = 16;
+// tokens of this step in order.  The key channels are cut into P slices of 4 (P a power of two, 4 P >= dim);
+// thread (e, p) keeps S[4 p .. 4 p + 3, e] in registers, and the P lanes of a column are neighbours, so the sum
+// over the channels ends with log2 P lane exchanges (moves inside a row of 16 lanes, then lane swaps).  The
+// order of additions is the same whatever the step holds.  Per token a thread's chain is one multiply-add a
+// state element; a head's columns are shared out over V / EC workgroups, so that one long prompt still fills
+// many compute units.  r, k and the decays of 16 tokens at a time are staged in LDS, the next 16 requested
+// before these are worked on.  In memory S lies as [head][s][e][p] (s the index within a slice): a wave's
+// accesses to the state are contiguous.
+constexpr int kSlice = 4;
 constexpr int kChunk = 16;
 
+template <int P>
+__device__ __forceinline__ float sum_over_slices(float v) {
+  if constexpr (P >= 2) v += dpp_f32<TL_DPP_XOR1>(v);
+  if constexpr (P >= 4) v += dpp_f32<TL_DPP_XOR2>(v);
+  if constexpr (P >= 8) v += dpp_f32<TL_DPP_HALF_MIRROR>(v);      // the quads of a half row hold one value each by now
+  if constexpr (P >= 16) v += dpp_f32<TL_DPP_MIRROR>(v);
+  if constexpr (P >= 32) {
+    float a, b;
+    pair16(v, a, b);
+    v = a + b;
+  }
+  if constexpr (P >= 64) {
+    float a, b;
+    pair32(v, a, b);
+    v = a + b;
+  }
+  return v;
+}
+
+template <int P>
 __global__ __launch_bounds__(kThreads) void time_mix_recurrence_kernel(
     const float* __restrict__ x, int64_t x_stride, int r_off, int k_off, int v_off, int w_off,
     const float* __restrict__ w0, const float* __restrict__ u, float* __restrict__ state, int64_t state_stride,
-    const int32_t* __restrict__ cu, const int32_t* __restrict__ slots, float* __restrict__ o, int heads, int dim, int vdim,
-    int P) {
-  extern __shared__ __align__(16) float lds[];
-  const int EC = kThreads / P, Dp = kSlice * P;
-  float* r_s = lds;                       // [kChunk][Dp]
-  float* k_s = r_s + kChunk * Dp;
-  float* w_s = k_s + kChunk * Dp;
-  float* v_s = w_s + kChunk * Dp;         // [kChunk][EC]
+    const int32_t* __restrict__ cu, const int32_t* __restrict__ slots, float* __restrict__ o, int heads, int dim, int vdim) {
+  constexpr int EC = kThreads / P, Dp = kSlice * P;
+  constexpr int NST = (kChunk * Dp + kThreads - 1) / kThreads, NV = (kChunk * EC + kThreads - 1) / kThreads;
+  __shared__ __align__(16) float r_s[kChunk * Dp];
+  __shared__ __align__(16) float k_s[kChunk * Dp];
+  __shared__ __align__(16) float w_s[kChunk * Dp];
+  __shared__ float v_s[kChunk * EC];
   const int req = blockIdx.z, head = blockIdx.y;
   const int t0 = cu[req], n = cu[req + 1] - t0;
   if (n <= 0) return;                     // a request without tokens touches no state
@@ -82,45 +104,68 @@ __global__ __launch_bounds__(kThreads) void time_mix_recurrence_kernel(
     const int d = p * kSlice + s;
     uu[s] = d < dim ? u[head * dim + d] : 0.f;
   }
+  // what this thread stages of a chunk: element i = tid + j * kThreads of [token][channel], token i / Dp
+  float pr[NST], pk[NST], pw[NST], pv[NV];
+  auto fetch = [&](int c0) {
+    const int m = min(kChunk, n - c0);
+#pragma unroll
+    for (int j = 0; j < NST; ++j) {
+      const int i = tid + j * kThreads, tt = i / Dp, d = i % Dp;
+      pr[j] = pk[j] = 0.f;
+      pw[j] = -INFINITY;                   // a channel beyond the head's: decay exp(-exp(-inf)) = 1, nothing added
+      if (i < kChunk * Dp && tt < m && d < dim) {
+        const float* row = x + (int64_t)(t0 + c0 + tt) * x_stride + head * dim + d;
+        pr[j] = row[r_off];
+        pk[j] = row[k_off];
+        pw[j] = row[w_off] + w0[head * dim + d];
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const int i = tid + j * kThreads, tt = i / EC, ee = blockIdx.x * EC + i % EC;
+      pv[j] = (i < kChunk * EC && tt < m && ee < vdim) ? x[(int64_t)(t0 + c0 + tt) * x_stride + v_off + head * vdim + ee] : 0.f;
+    }
+  };
+  fetch(0);
   for (int c0 = 0; c0 < n; c0 += kChunk) {
     const int m = min(kChunk, n - c0);
-    __syncthreads();
-    for (int i = tid; i < m * Dp; i += kThreads) {
-      const int tt = i / Dp, d = i - tt * Dp;
-      float rr = 0.f, kk = 0.f, ww = 1.f;
-      if (d < dim) {
-        const float* row = x + (int64_t)(t0 + c0 + tt) * x_stride + head * dim + d;
-        rr = row[r_off];
-        kk = row[k_off];
-        ww = expf(-expf(row[w_off] + w0[head * dim + d]));
+    __syncthreads();                       // the chunk before is done with
+#pragma unroll
+    for (int j = 0; j < NST; ++j) {
+      const int i = tid + j * kThreads;
+      if (i < kChunk * Dp) {
+        r_s[i] = pr[j];
+        k_s[i] = pk[j];
+        w_s[i] = expf(-expf(pw[j]));
       }
-      r_s[i] = rr;
-      k_s[i] = kk;
-      w_s[i] = ww;
     }
-    for (int i = tid; i < m * EC; i += kThreads) {
-      const int tt = i / EC, ee = blockIdx.x * EC + (i - tt * EC);
-      v_s[i] = ee < vdim ? x[(int64_t)(t0 + c0 + tt) * x_stride + v_off + head * vdim + ee] : 0.f;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const int i = tid + j * kThreads;
+      if (i < kChunk * EC) v_s[i] = pv[j];
     }
     __syncthreads();
-    for (int tt = 0; tt < m; ++tt) {
+    if (c0 + kChunk < n) fetch(c0 + kChunk);      // on its way while this chunk is worked on
+    float* orow = o + (int64_t)(t0 + c0) * ((int64_t)heads * vdim) + head * vdim + e;
+    auto token = [&](int tt) {
       const float vv = v_s[tt * EC + el];
-      const float* rp = r_s + tt * Dp + p * kSlice;
-      const float* kp = k_s + tt * Dp + p * kSlice;
-      const float* wp = w_s + tt * Dp + p * kSlice;
+      const f32x4 r4 = *(const f32x4*)(r_s + tt * Dp + p * kSlice), k4 = *(const f32x4*)(k_s + tt * Dp + p * kSlice),
+                  w4 = *(const f32x4*)(w_s + tt * Dp + p * kSlice);
       float acc = 0.f;
 #pragma unroll
-      for (int s4 = 0; s4 < kSlice; s4 += 4) {
-        const f32x4 r4 = *(const f32x4*)(rp + s4), k4 = *(const f32x4*)(kp + s4), w4 = *(const f32x4*)(wp + s4);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const float kv = k4[j] * vv;
-          acc = fmaf(r4[j], fmaf(uu[s4 + j], kv, S[s4 + j]), acc);
-          S[s4 + j] = fmaf(w4[j], S[s4 + j], kv);
-        }
+      for (int j = 0; j < kSlice; ++j) {
+        const float kv = k4[j] * vv;
+        acc = fmaf(r4[j], fmaf(uu[j], kv, S[j]), acc);
+        S[j] = fmaf(w4[j], S[j], kv);
       }
-      for (int sh = P >> 1; sh >= 1; sh >>= 1) acc += __shfl_xor(acc, sh, TL_WAVE);
-      if (p == 0 && col) o[(int64_t)(t0 + c0 + tt) * ((int64_t)heads * vdim) + head * vdim + e] = acc;
+      acc = sum_over_slices<P>(acc);
+      if (p == 0 && col) orow[(int64_t)tt * heads * vdim] = acc;
+    };
+    if (m == kChunk) {
+#pragma unroll
+      for (int tt = 0; tt < kChunk; ++tt) token(tt);
+    } else {
+      for (int tt = 0; tt < m; ++tt) token(tt);
     }
   }
   if (col) {
@@ -184,7 +229,7 @@ int tl_shift_save(const void* h, int64_t h_stride, float* state, int64_t state_s
 }
 
 // x: float32 rows that hold r, k, the decay's pre-activation (heads * dim columns each, from r_off, k_off, w_off)
-// and v (heads * vdim columns from v_off).  state rows: S as [heads][16][vdim][P] floats from column 0, P =
+// and v (heads * vdim columns from v_off).  state rows: S as [heads][4][vdim][P] floats from column 0, P =
 // tl_time_mix_slices(dim).  o: float32 [n_tokens, heads * vdim].
 int tl_time_mix_recurrence(const float* x, int64_t x_stride, int r_off, int k_off, int v_off, int w_off, const float* w0,
                            const float* u, float* state, int64_t state_stride, const int32_t* cu, const int32_t* slots,
@@ -196,10 +241,18 @@ int tl_time_mix_recurrence(const float* x, int64_t x_stride, int r_off, int k_of
   const int P = tl_time_mix_slices(dim);
   if (state_stride < (int64_t)heads * kSlice * vdim * P) return TL_ERR_ARG;
   const int EC = kThreads / P;
-  const size_t smem = (size_t)kChunk * (3 * kSlice * P + EC) * sizeof(float);
+  if ((vdim + EC - 1) / EC > 65535) return TL_ERR_ARG;
   dim3 g((vdim + EC - 1) / EC, heads, n_requests), b(kThreads);
-  hipLaunchKernelGGL(time_mix_recurrence_kernel, g, b, smem, stream, x, x_stride, r_off, k_off, v_off, w_off, w0, u, state,
-                     state_stride, cu, slots, o, heads, dim, vdim, P);
+#define TL_TIME_MIX(PP)                                                                                               \
+  case PP:                                                                                                            \
+    hipLaunchKernelGGL(time_mix_recurrence_kernel<PP>, g, b, 0, stream, x, x_stride, r_off, k_off, v_off, w_off, w0, u, \
+                       state, state_stride, cu, slots, o, heads, dim, vdim);                                          \
+    break;
+  switch (P) {
+    TL_TIME_MIX(1) TL_TIME_MIX(2) TL_TIME_MIX(4) TL_TIME_MIX(8) TL_TIME_MIX(16) TL_TIME_MIX(32) TL_TIME_MIX(64)
+    default: return TL_ERR_ARG;
+  }
+#undef TL_TIME_MIX
   return tl_launch_status();
 }
 

@@ -1658,11 +1658,11 @@ def gelu_glu(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
 
 # -------------------------------------------------------- time mixing with a decaying state
 TIME_MIX_MAX_DIM = 256      # key channels of a head (csrc/time_mix.hip)
-TIME_MIX_SLICE = 16
+TIME_MIX_SLICE = 4
 
 
 def time_mix_slices(dim: int) -> int:
-    """Slices of 16 key channels a head's state is cut into (a power of two)."""
+    """Slices of 4 key channels a head's state is cut into (a power of two)."""
     p = 1
     while p * TIME_MIX_SLICE < dim:
         p *= 2
@@ -1797,28 +1797,105 @@ def table_moe_down(z: torch.Tensor, w: torch.Tensor, tokens: torch.Tensor, table
 MOE_TILE_ROWS = 32          # rows of one expert a tile of the grouped product holds (csrc/moe.hip)
 
 
-def moe_max_tiles(rows: int, experts: int) -> int:
-    return -(-rows // MOE_TILE_ROWS) + experts
+MOE_RUN_ROWS = 256          # rows of one expert a run of the tiled product's rows holds (a multiple of its tile heights)
 
 
-def moe_plan_ints(rows: int, experts: int) -> int:
+def moe_max_tiles(rows: int, experts: int, tile_rows: int = MOE_TILE_ROWS) -> int:
+    return -(-rows // tile_rows) + experts
+
+
+def moe_plan_ints(rows: int, experts: int, tile_rows: int = MOE_TILE_ROWS) -> int:
     """int32 elements of the plan `moe_plan` fills for `rows` (= tokens * top) rows."""
-    return 3 * experts + 2 + 3 * moe_max_tiles(rows, experts) + rows
+    return 3 * experts + 2 + 3 * moe_max_tiles(rows, experts, tile_rows) + rows
 
 
-def moe_plan(tokens: torch.Tensor, table: torch.Tensor, plan: torch.Tensor, experts: int) -> torch.Tensor:
+def moe_plan(tokens: torch.Tensor, table: torch.Tensor, plan: torch.Tensor, experts: int,
+             tile_rows: int = MOE_TILE_ROWS) -> torch.Tensor:
     """Sorts the step's rows (token t, its j-th expert: row t * top + j) by expert on the device and lists
-    tiles of at most 32 rows of one expert each; `plan` is int32 scratch of `moe_plan_ints` elements."""
+    tiles of at most `tile_rows` rows of one expert each; `plan` is int32 scratch of `moe_plan_ints` elements:
+    counts[E], cursors[E], offsets[E + 1], the number of tiles, then per tile (capacity `moe_max_tiles`) its
+    expert (-1 behind the last tile), its first place in the sorted rows and its number of rows, then the rows
+    sorted by expert."""
     _dev(tokens, table, plan)
     _i32(tokens, table, plan)
     V, top = table.shape
     T = tokens.numel()
-    _need(plan.numel() >= moe_plan_ints(T * top, experts), "moe_plan: the plan is too short")
+    _need(plan.numel() >= moe_plan_ints(T * top, experts, tile_rows), "moe_plan: the plan is too short")
     _need(0 < experts <= 1024, "moe_plan: 1 to 1024 experts")
     plan[:2 * experts].zero_()          # counts and cursors (a fill kernel: fine inside a captured step)
     _check(_lib().tl_moe_plan(_ptr(tokens), _ptr(table), _ptr(plan), c_int(T), c_int(top), c_int(experts), c_int(V),
-                              c_int(moe_max_tiles(T * top, experts)), _stream()), "moe_plan")
+                              c_int(moe_max_tiles(T * top, experts, tile_rows)), c_int(tile_rows), _stream()), "moe_plan")
     return plan
+
+
+def moe_tile_experts(plan: torch.Tensor, rows: int, experts: int, tile_rows: int) -> torch.Tensor:
+    """The plan's list of experts by tile (-1: the tile holds no row)."""
+    at = 3 * experts + 2
+    return plan[at:at + moe_max_tiles(rows, experts, tile_rows)]
+
+
+def moe_gather(a: Optional[torch.Tensor], a_div: int, plan: torch.Tensor, rows: int, experts: int, tile_rows: int,
+               dst: Optional[torch.Tensor], row_pos: Optional[torch.Tensor]) -> None:
+    """The plan's rows side by side, a tile after the other: dst[tile * tile_rows + i] = a[row // a_div] (bfloat16;
+    a None: nothing is copied) and row_pos[row] = tile * tile_rows + i (int32 [rows]; None: not wanted)."""
+    _dev(a, plan, dst, row_pos)
+    _i32(plan)
+    mt = moe_max_tiles(rows, experts, tile_rows)
+    _need(plan.numel() >= moe_plan_ints(rows, experts, tile_rows), "moe_gather: the plan is too short")
+    K = 8
+    if a is not None:
+        _rows_2d(a, "moe_gather input")
+        K = a.shape[1]
+        _need(a.dtype == torch.bfloat16 and dst is not None and dst.dtype == torch.bfloat16 and dst.is_contiguous()
+              and tuple(dst.shape) == (mt * tile_rows, K) and K % 8 == 0 and a.stride(0) % 8 == 0
+              and a.shape[0] * a_div >= rows, "moe_gather: a [*, K] and contiguous dst [tiles * tile_rows, K] are bfloat16")
+    if row_pos is not None:
+        _i32(row_pos)
+        _need(row_pos.numel() >= rows, "moe_gather: one place per row")
+    _check(_lib().tl_moe_gather(_ptr(a, 16), c_int64(a.stride(0) if a is not None else 0), c_int(a_div), _ptr(dst, 16),
+                                _ptr(row_pos), _ptr(plan), c_int(experts), c_int(mt), c_int(tile_rows), c_int(K),
+                                _stream()), "moe_gather")
+
+
+def linear_grouped(a: torch.Tensor, w: torch.Tensor, tile_group: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out = a @ w[g]^T by runs of 256 rows: run r of a (bfloat16 [runs * 256, K]) multiplies w[tile_group[r]]
+    (bfloat16 [G, N, K]); a run whose entry is negative is skipped (its rows of out are not written).  out
+    [runs * 256, N] bfloat16 or float32.  The tiled product of `linear` with a weight matrix per run of rows."""
+    _dev(a, w, tile_group, out)
+    _rows_2d(a, "linear_grouped input")
+    _rows_2d(out, "linear_grouped output")
+    M, K = a.shape
+    G, N, _ = w.shape
+    _need(a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and w.is_contiguous() and w.shape[2] == K,
+          "linear_grouped: a [M, K] and contiguous w [G, N, K] are bfloat16")
+    _need(M % MOE_RUN_ROWS == 0 and K % 8 == 0 and a.stride(0) % 8 == 0, "linear_grouped: runs of 256 rows, K a multiple of 8")
+    _need(tuple(out.shape) == (M, N), "linear_grouped: out is [M, N]")
+    _i32(tile_group)
+    _need(tile_group.numel() >= M // MOE_RUN_ROWS, "linear_grouped: one group per run of rows")
+    _check(_lib().tl_linear_grouped(_ptr(a, 16), _ptr(w, 16), _ptr(out, 16), _ptr(tile_group), c_int(MOE_RUN_ROWS),
+                                    c_int(M), c_int(N), c_int(K), c_int64(a.stride(0)), c_int64(out.stride(0)),
+                                    c_int(_dt(out)), _stream()), "linear_grouped")
+    return out
+
+
+def moe_combine_at(y: torch.Tensor, row_pos: torch.Tensor, out: torch.Tensor, top: int, coef: float,
+                   base: Optional[torch.Tensor] = None, base_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[t] = base[t] * base_scale[t] + coef * sum_j y[row_pos[t * top + j]]; y float32 [*, N], out float32 [T, N]."""
+    _dev(y, row_pos, out, base, base_scale)
+    T, N = out.shape
+    _need(out.dtype == torch.float32 and out.is_contiguous(), "moe_combine_at: out is contiguous float32 [T, N]")
+    _need(y.dtype == torch.float32 and y.is_contiguous() and y.dim() == 2 and y.shape[1] == N,
+          "moe_combine_at: y is contiguous float32 [*, N]")
+    _i32(row_pos)
+    _need(row_pos.numel() >= T * top, "moe_combine_at: one place per row")
+    if base is not None:
+        _need(base.dtype == torch.float32 and base.is_contiguous() and base.shape == out.shape,
+              "moe_combine_at: base is contiguous float32 [T, N]")
+    if base_scale is not None:
+        _f32_vec(base_scale, T, "moe_combine_at base_scale")
+    _check(_lib().tl_moe_combine_at(_ptr(y), _ptr(row_pos), _ptr(base), _ptr(base_scale), _ptr(out), c_int(T), c_int(N),
+                                    c_int(top), c_float(coef), _stream()), "moe_combine_at")
+    return out
 
 
 def grouped_rows_gemm(a: torch.Tensor, a_div: int, w: torch.Tensor, plan: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
@@ -1834,7 +1911,7 @@ def grouped_rows_gemm(a: torch.Tensor, a_div: int, w: torch.Tensor, plan: torch.
     _need(out.is_contiguous() and out.shape[1] == N and a.shape[0] * a_div >= rows,
           "grouped_rows_gemm: out is contiguous [rows, N], a holds rows / a_div rows")
     _i32(plan)
-    _need(plan.numel() >= moe_plan_ints(rows, E), "grouped_rows_gemm: the plan is too short")
+    _need(plan.numel() >= moe_plan_ints(rows, E), "grouped_rows_gemm: the plan is too short (tiles of 32 rows)")
     _check(_lib().tl_grouped_rows_gemm(_ptr(a, 16), c_int64(a.stride(0)), c_int(a_div), _ptr(w, 16), _ptr(out),
                                        _ptr(plan), c_int(rows), c_int(E), c_int(moe_max_tiles(rows, E)), c_int(N),
                                        c_int(K), c_int(_dt(out)), _stream()), "grouped_rows_gemm")

@@ -21,6 +21,7 @@ from .mlp import ClampedGLU
 class TableMoE(FeedForward):
     graph_safe = True
     GROUPED_ROWS = 64       # from this many rows (tokens * top) on, a bfloat16 step groups its rows by expert
+    RUN_ROWS = 64           # from this many rows an expert on average, the rows are copied into runs of 256 an expert
 
     def __init__(self, prefix, dtype, device, *, hidden_size: int, vocab_size: int, num_experts: int, top: int,
                  intermediate_size: int, limit: float, alpha: float = 1.702, shift: float = 1.0,
@@ -81,11 +82,29 @@ class TableMoE(FeedForward):
             if self.shared_gate:
                 scale = ops.row_dot_sigmoid(h, self.w_sg, ops.scratch("moe_shared_gate", (T,), torch.float32, dev))
         rows = T * self.top
-        gu = ops.scratch("moe_gate_up", (rows, 2 * F), self.dtype, dev)
-        z = ops.scratch("moe_gated", (rows, F), self.dtype, dev)
         out = base if base is not None else ops.scratch("sublayer_out", (T, self.hidden_size), torch.float32, dev)
-        if self.dtype == torch.bfloat16 and rows >= self.GROUPED_ROWS:
+        if self.dtype == torch.bfloat16 and rows >= self.RUN_ROWS * self.num_experts:
+            # very many rows (prompts): every expert's rows side by side in runs of 256, and the tiled product of
+            # the dense layers with a weight matrix per run
+            E, R = self.num_experts, ops.MOE_RUN_ROWS
+            cap = ops.moe_max_tiles(rows, E, R) * R
+            plan = ops.scratch("moe_plan", (ops.moe_plan_ints(rows, E, R),), torch.int32, dev)
+            ops.moe_plan(tokens, self.table, plan, E, R)
+            runs = ops.moe_tile_experts(plan, rows, E, R)
+            hp = ops.scratch("moe_rows_in", (cap, self.hidden_size), self.dtype, dev)
+            pos = ops.scratch("moe_row_pos", (rows,), torch.int32, dev)
+            ops.moe_gather(h, self.top, plan, rows, E, R, hp, pos)
+            gup = ops.scratch("moe_gate_up", (cap, 2 * F), self.dtype, dev)
+            ops.linear_grouped(hp, self.w_gate_up, runs, gup)
+            zp = ops.scratch("moe_gated", (cap, F), self.dtype, dev)
+            ops.clamped_glu(gup, zp, self.limit, self.alpha, self.shift)
+            y = ops.scratch("moe_rows_out", (cap, self.hidden_size), torch.float32, dev)
+            ops.linear_grouped(zp, self.w_down, runs, y)
+            ops.moe_combine_at(y, pos, out, self.top, 1.0 / self.top, base, scale)
+        elif self.dtype == torch.bfloat16 and rows >= self.GROUPED_ROWS:
             # many rows: sorted by expert on the device, tiles of one expert's rows on the matrix cores
+            gu = ops.scratch("moe_gate_up", (rows, 2 * F), self.dtype, dev)
+            z = ops.scratch("moe_gated", (rows, F), self.dtype, dev)
             plan = ops.scratch("moe_plan", (ops.moe_plan_ints(rows, self.num_experts),), torch.int32, dev)
             ops.moe_plan(tokens, self.table, plan, self.num_experts)
             ops.grouped_rows_gemm(h, self.top, self.w_gate_up, plan, gu)
@@ -95,6 +114,8 @@ class TableMoE(FeedForward):
             ops.moe_combine(y, out, self.top, 1.0 / self.top, base, scale)
         else:
             # few rows (decoding) and float32: each row against its own expert's weights
+            gu = ops.scratch("moe_gate_up", (rows, 2 * F), self.dtype, dev)
+            z = ops.scratch("moe_gated", (rows, F), self.dtype, dev)
             ops.table_moe_up(h, self.w_gate_up, tokens, self.table, gu)
             ops.clamped_glu(gu, z, self.limit, self.alpha, self.shift)
             ops.table_moe_down(z, self.w_down, tokens, self.table, out, 1.0 / self.top, base, scale)
