@@ -424,7 +424,7 @@ def test_time_mix_state_over_slots_and_tiny_portions(H, D):
     for s in slots:
         state[s].zero_()
     at, got_o, got_mix = [0, 0, 0], [[], [], []], [[], [], []]
-    sizes = [3, 1, 7, 2, 1, 5, 2, 6]
+    sizes = [3, 1, 7, 2, 1, 5, 2, 6, 1, 1, 1, 1, 1, 1]
     k = 0
     while any(a < n for a, n in zip(at, lens)):
         live = [r for r in (2, 0, 1) if at[r] < lens[r]]             # batch order differs from slot order
@@ -439,8 +439,10 @@ def test_time_mix_state_over_slots_and_tiny_portions(H, D):
         req = torch.tensor([i for i, m in enumerate(take) for _ in range(m)], dtype=torch.int32, device=dev)
         sl = torch.tensor([slots[r] for r in live], dtype=torch.int32, device=dev)
         mixes = torch.empty(2, T, W, device=dev)
-        ops.shift_mix(h, state, s_floats, req, cu, sl, mu.to(dev), mixes)
-        ops.shift_save(h, state, s_floats, cu, sl)
+        single = all(m == 1 for m in take)            # such a step's shift saves the tokens itself
+        ops.shift_mix(h, state, s_floats, req, cu, sl, mu.to(dev), mixes, save_single=single)
+        if not single:
+            ops.shift_save(h, state, s_floats, cu, sl)
         o = torch.empty(T * S, device=dev)
         ops.time_mix_recurrence(x, 0, S, 2 * S, 3 * S, w0.to(dev), u.reshape(-1).to(dev), state, cu, sl, o, H, D, D)
         o = o.reshape(T, H, D).cpu()

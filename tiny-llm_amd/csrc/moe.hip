@@ -42,6 +42,65 @@ __device__ __forceinline__ float dot_lanes(const bf16_t* __restrict__ a, const b
   return wave_sum(acc);
 }
 
+// Four dot products of one row at once (the loads of four weight rows in flight together); each sum is formed
+// exactly as dot_lanes forms it.
+__device__ __forceinline__ void dot_lanes4(const float* __restrict__ a, const float* const* w, int K, int lane, float* out) {
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  bool vec = (K & 3) == 0 && (((uintptr_t)a) & 15) == 0;
+#pragma unroll
+  for (int c = 0; c < 4; ++c) vec = vec && (((uintptr_t)w[c]) & 15) == 0;
+  if (vec) {
+    for (int k = lane * 4; k < K; k += TL_WAVE * 4) {
+      const f32x4 x = *(const f32x4*)(a + k);
+      f32x4 y[4];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) y[c] = *(const f32x4*)(w[c] + k);
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        acc[c] = fmaf(x[0], y[c][0], acc[c]);
+        acc[c] = fmaf(x[1], y[c][1], acc[c]);
+        acc[c] = fmaf(x[2], y[c][2], acc[c]);
+        acc[c] = fmaf(x[3], y[c][3], acc[c]);
+      }
+    }
+  } else {
+    for (int k = lane; k < K; k += TL_WAVE) {
+      const float x = a[k];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) acc[c] = fmaf(x, w[c][k], acc[c]);
+    }
+  }
+#pragma unroll
+  for (int c = 0; c < 4; ++c) out[c] = wave_sum(acc[c]);
+}
+
+__device__ __forceinline__ void dot_lanes4(const bf16_t* __restrict__ a, const bf16_t* const* w, int K, int lane, float* out) {
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  bool vec = (K & 7) == 0 && (((uintptr_t)a) & 15) == 0;
+#pragma unroll
+  for (int c = 0; c < 4; ++c) vec = vec && (((uintptr_t)w[c]) & 15) == 0;
+  if (vec) {
+    for (int k = lane * 8; k < K; k += TL_WAVE * 8) {
+      const bf16x8 x = *(const bf16x8*)(a + k);
+      bf16x8 y[4];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) y[c] = *(const bf16x8*)(w[c] + k);
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[c] = fmaf((float)x[j], (float)y[c][j], acc[c]);
+    }
+  } else {
+    for (int k = lane; k < K; k += TL_WAVE) {
+      const float x = (float)a[k];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) acc[c] = fmaf(x, (float)w[c][k], acc[c]);
+    }
+  }
+#pragma unroll
+  for (int c = 0; c < 4; ++c) out[c] = wave_sum(acc[c]);
+}
+
 __device__ __forceinline__ int expert_of(const int32_t* tokens, const int32_t* table, int t, int j, int top, int vocab,
                                          int experts) {
   int tok = tokens[t];
@@ -63,9 +122,13 @@ __global__ __launch_bounds__(kThreads) void table_moe_up_kernel(const T* __restr
   const T* arow = a + (int64_t)t * a_stride;
   const T* we = w + (int64_t)e * N * K;
   const int n0 = blockIdx.y * kCols + wave * (kCols / kWaves);
-  for (int n = n0; n < min(N, n0 + kCols / kWaves); ++n) {
-    const float v = dot_lanes(arow, we + (int64_t)n * K, K, lane);
-    if (lane == 0) out[(int64_t)row * N + n] = from_f32<T>(v);
+  for (int n = n0; n < min(N, n0 + kCols / kWaves); n += 4) {
+    const T* wr[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) wr[c] = we + (int64_t)min(n + c, N - 1) * K;
+    float v[4];
+    dot_lanes4(arow, wr, K, lane, v);
+    if (lane < 4 && n + lane < N) out[(int64_t)row * N + n + lane] = from_f32<T>(v[lane]);
   }
 }
 
@@ -83,15 +146,21 @@ __global__ __launch_bounds__(kThreads) void table_moe_down_kernel(const T* __res
   const int wave = threadIdx.x / TL_WAVE, lane = threadIdx.x % TL_WAVE;
   const int n0 = blockIdx.y * kCols + wave * (kCols / kWaves);
   const float bsc = base_scale ? base_scale[t] : 1.f;
-  for (int n = n0; n < min(N, n0 + kCols / kWaves); ++n) {
-    float acc = 0.f;
+  for (int n = n0; n < min(N, n0 + kCols / kWaves); n += 4) {
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
     for (int j = 0; j < top; ++j) {
       const int e = expert_of(tokens, table, t, j, top, vocab, experts);
-      acc += dot_lanes(z + ((int64_t)t * top + j) * K, w + ((int64_t)e * N + n) * K, K, lane);
+      const T* wr[4];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) wr[c] = w + ((int64_t)e * N + min(n + c, N - 1)) * K;
+      float v[4];
+      dot_lanes4(z + ((int64_t)t * top + j) * K, wr, K, lane, v);
+#pragma unroll
+      for (int c = 0; c < 4; ++c) acc[c] += v[c];
     }
-    if (lane == 0) {
-      const float b = base ? base[(int64_t)t * N + n] * bsc : 0.f;
-      out[(int64_t)t * N + n] = fmaf(coef, acc, b);
+    if (lane < 4 && n + lane < N) {
+      const float b = base ? base[(int64_t)t * N + n + lane] * bsc : 0.f;
+      out[(int64_t)t * N + n + lane] = fmaf(coef, acc[lane], b);
     }
   }
 }

@@ -20,15 +20,22 @@ __global__ __launch_bounds__(kThreads) void shift_mix_kernel(const T* __restrict
                                                              const int32_t* __restrict__ cu,
                                                              const int32_t* __restrict__ slots,
                                                              const float* __restrict__ mu, T* __restrict__ out,
-                                                             int64_t plane, int n_mix, int width) {
+                                                             int64_t plane, int n_mix, int width, int save_single) {
   const int t = blockIdx.x;
   const int c = blockIdx.y * kThreads + threadIdx.x;
   if (c >= width) return;
   const int r = req_of_token[t];
   const float cur = to_f32(h[(int64_t)t * h_stride + c]);
   float prev;
-  if (t == cu[r]) prev = state[(int64_t)slots[r] * state_stride + prev_off + c];
-  else prev = to_f32(h[(int64_t)(t - 1) * h_stride + c]);
+  if (t == cu[r]) {
+    float* saved = const_cast<float*>(state) + (int64_t)slots[r] * state_stride + prev_off + c;
+    prev = *saved;
+    // a request's only token of the step is also its last: this thread has read what the state kept and leaves
+    // the token's h in its place (steps of single tokens then need no kernel of their own for that)
+    if (save_single && cu[r + 1] == t + 1) *saved = cur;
+  } else {
+    prev = to_f32(h[(int64_t)(t - 1) * h_stride + c]);
+  }
   const float d = prev - cur;
   for (int m = 0; m < n_mix; ++m)
     out[(int64_t)m * plane + (int64_t)t * width + c] = from_f32<T>(fmaf(d, mu[(int64_t)m * width + c], cur));
@@ -194,19 +201,21 @@ int tl_time_mix_slices(int dim) {
 }
 
 // h: [n_tokens, width] of the engine's type; mu: float32 [n_mix, width]; out: [n_mix, n_tokens, width].
-int tl_shift_mix(const void* h, int64_t h_stride, const float* state, int64_t state_stride, int64_t prev_off,
+// save_single: a request that brings exactly one token also gets that token's h saved in its state row (requests
+// with more tokens need tl_shift_save behind this kernel).
+int tl_shift_mix(const void* h, int64_t h_stride, float* state, int64_t state_stride, int64_t prev_off,
                  const int32_t* req_of_token, const int32_t* cu, const int32_t* slots, const float* mu, void* out,
-                 int n_tokens, int n_mix, int width, int dtype, hipStream_t stream) {
+                 int n_tokens, int n_mix, int width, int save_single, int dtype, hipStream_t stream) {
   if (n_tokens <= 0) return TL_OK;
   if (width <= 0 || n_mix <= 0 || !h || !state || !req_of_token || !cu || !slots || !mu || !out) return TL_ERR_ARG;
   dim3 g(n_tokens, (width + kThreads - 1) / kThreads), b(kThreads);
   const int64_t plane = (int64_t)n_tokens * width;
   if (dtype == 0)
     hipLaunchKernelGGL(shift_mix_kernel<float>, g, b, 0, stream, (const float*)h, h_stride, state, state_stride, prev_off,
-                       req_of_token, cu, slots, mu, (float*)out, plane, n_mix, width);
+                       req_of_token, cu, slots, mu, (float*)out, plane, n_mix, width, save_single);
   else if (dtype == 1)
     hipLaunchKernelGGL(shift_mix_kernel<bf16_t>, g, b, 0, stream, (const bf16_t*)h, h_stride, state, state_stride,
-                       prev_off, req_of_token, cu, slots, mu, (bf16_t*)out, plane, n_mix, width);
+                       prev_off, req_of_token, cu, slots, mu, (bf16_t*)out, plane, n_mix, width, save_single);
   else
     return TL_ERR_ARG;
   return tl_launch_status();

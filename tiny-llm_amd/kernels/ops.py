@@ -1675,9 +1675,11 @@ def time_mix_state_floats(heads: int, dim: int, vdim: int) -> int:
 
 
 def shift_mix(h: torch.Tensor, state: torch.Tensor, prev_off: int, req_of_token: torch.Tensor, cu_seqlens: torch.Tensor,
-              state_slots: torch.Tensor, mu: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+              state_slots: torch.Tensor, mu: torch.Tensor, out: torch.Tensor, save_single: bool = False) -> torch.Tensor:
     """out[m, t] = h[t] + (h[t - 1] - h[t]) * mu[m]; for the first token a request brings in this step h[t - 1] is what
-    its state row keeps at prev_off.  h [T, W] and out [M, T, W] of one type, mu float32 [M, W], state float32 rows."""
+    its state row keeps at prev_off.  h [T, W] and out [M, T, W] of one type, mu float32 [M, W], state float32 rows.
+    save_single: a request that brings exactly one token gets it saved as `shift_save` would (a step in which no
+    request brings more needs no `shift_save` then)."""
     _dev(h, state, req_of_token, cu_seqlens, state_slots, mu, out)
     _rows_2d(h, "shift_mix input")
     T, W = h.shape
@@ -1688,10 +1690,11 @@ def shift_mix(h: torch.Tensor, state: torch.Tensor, prev_off: int, req_of_token:
     _need(state.dtype == torch.float32 and state.dim() == 2 and state.stride(1) == 1 and state.shape[1] >= prev_off + W,
           "shift_mix: state rows are float32 and hold W values from prev_off")
     _i32(req_of_token, cu_seqlens, state_slots)
-    _need(req_of_token.numel() == T, "shift_mix: one request index per token")
+    _need(req_of_token.numel() == T and cu_seqlens.numel() == state_slots.numel() + 1,
+          "shift_mix: one request index per token, cu_seqlens one entry more than there are requests")
     _check(_lib().tl_shift_mix(_ptr(h), c_int64(h.stride(0)), _ptr(state), c_int64(state.stride(0)), c_int64(prev_off),
                                _ptr(req_of_token), _ptr(cu_seqlens), _ptr(state_slots), _ptr(mu), _ptr(out), c_int(T),
-                               c_int(M), c_int(W), c_int(_dt(h)), _stream()), "shift_mix")
+                               c_int(M), c_int(W), c_int(1 if save_single else 0), c_int(_dt(h)), _stream()), "shift_mix")
     return out
 
 

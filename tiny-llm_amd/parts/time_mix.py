@@ -83,8 +83,11 @@ class TimeMix(Mixer):
     def forward(self, h, ctx, cache, state, residual):
         T, dev, S, seg = h.shape[0], h.device, self.size, self.seg
         mixes = ops.scratch("shift_mixes", (len(self.MIXES), T, self.hidden_size), self.dtype, dev)
-        ops.shift_mix(h, state, self.s_floats, ctx.req_of_token, ctx.cu_seqlens_q, ctx.state_slots, self.mu, mixes)
-        ops.shift_save(h, state, self.s_floats, ctx.cu_seqlens_q, ctx.state_slots)
+        single = ctx.max_q_len == 1              # no request brings more than one token: the shift saves it itself
+        ops.shift_mix(h, state, self.s_floats, ctx.req_of_token, ctx.cu_seqlens_q, ctx.state_slots, self.mu, mixes,
+                      save_single=single)
+        if not single:
+            ops.shift_save(h, state, self.s_floats, ctx.cu_seqlens_q, ctx.state_slots)
         x = ops.scratch("time_mix_in", (T, 4 * seg), torch.float32, dev)
         ops.linear(mixes[0], self.w_r, x[:, 0:S])
         ops.linear(mixes[1], self.w_k, x[:, seg:seg + S])
