@@ -71,6 +71,42 @@ ONLY_MOE = model(64, 199, [layer(left(2, 2, 24, 9, 6), right(3, 24, 9), moe(4, 2
 CONFIGS = {"A": (MIX_A, 16), "B": (MIX_B, 8), "dense": (ONLY_DENSE, 4), "moe": (ONLY_MOE, 16)}
 
 
+def random_config(seed):
+    """A configuration drawn at random: width, vocabulary, two to four layers that each draw their own head
+    counts and sizes, window, rotated dims, time-mix shape, rank and feed-forward."""
+    import random
+    rng = random.Random(seed)
+    width = rng.choice([64, 96, 128, 192, 320])
+    vocab = rng.randrange(90, 700)
+    layers = []
+    for _ in range(rng.randrange(2, 5)):
+        dim = rng.choice([16, 24, 32, 48, 64, 80, 128])
+        kv = rng.choice([1, 2, 3])
+        heads = kv * rng.choice([1, 2, 3, 4])
+        while heads * dim % 8:
+            heads += kv
+        rot = rng.choice([0, dim, dim // 2 // 2 * 2, 2])
+        a = left(heads, kv, dim, rng.choice([1, 2, 5, 16, 31, 64, 100, 5000]), rot, rng.choice([100.0, 10000.0, 250000.0]),
+                 rng.choice([dim ** -0.5, 2.0 * dim ** -0.5, 4.0 / dim]))       # typical scores of a few units
+        td = rng.choice([8, 16, 24, 32, 40, 64, 96, 128])
+        th = rng.randrange(1, 5)
+        while th * td % 8:
+            th += 1
+        t = right(th, td, rng.choice([1, 4, 8, 13, 32]))
+        kind = rng.choice(["dense", "moe", "moe", "none"])
+        if kind == "dense":
+            mlp = dense(8 * rng.randrange(1, 40))
+        elif kind == "moe":
+            e = rng.randrange(1, 10)
+            shared = rng.choice([None, (8 * rng.randrange(1, 12), rng.uniform(0.5, 4.0), rng.random() < 0.7)])
+            mlp = moe(e, rng.randrange(1, e + 1), 8 * rng.randrange(1, 12), rng.uniform(0.5, 4.0), shared)
+        else:
+            mlp = None
+        layers.append(layer(a, t, mlp, rng.uniform(0.3, 1.6), rng.uniform(0.3, 1.6),
+                            norm2=(rng.random() < 0.5) if mlp is None else None))
+    return model(width, vocab, layers, alpha=rng.choice([0.5, 1.0, 2.5, 4.0]), eps=rng.choice([1e-5, 1e-6, 1e-4]))
+
+
 def random_weights(cfg, seed=0, sharpen=3.0):
     """{name: tensor} (float32; the experts' table int32).  `sharpen`: the gain of the projections that make
     scores, gates and decays (3: far from uniform, a misplaced key or a lost state moves the logits; 1: tame, so

@@ -126,6 +126,30 @@ def test_mixed_batches_reuse_pages_and_slots(name, dtype, tmp_path_factory):
         assert all_free(runner)
 
 
+@pytest.mark.parametrize("seed", range(10))
+def test_configurations_drawn_at_random(seed, tmp_path):
+    """Sizes nobody chose: width, heads and head sizes (with and without a matrix-core attention kernel), windows
+    from one token to more than the prompt, rotated dims, time-mix shapes, ranks, feed-forwards of every kind and
+    none, pages of 4 to 32 tokens; mixed batches and portions in both precisions against the plain model."""
+    import random
+    from fofapel_util import random_config
+    cfg = random_config(seed)
+    rng = random.Random(1000 + seed)
+    block = rng.choice([4, 8, 16, 32])
+    for dtype in ("float32", "bfloat16"):
+        folder, w = make_folder(tmp_path / dtype, cfg, seed=seed, store=torch.bfloat16 if dtype == "bfloat16" else torch.float32,
+                                sharpen=1.0 if dtype == "bfloat16" else 3.0)
+        w64 = rounded(w) if dtype == "bfloat16" else as_double(w)
+        reqs = {f"r{i}": random_tokens(n, cfg["vocab"], 7 * seed + i) for i, n in enumerate([rng.randrange(1, 140) for _ in range(5)])}
+        ref = {rid: plain.forward(cfg, w64, toks) for rid, toks in reqs.items()}
+        steps, peak = traces.mixed(reqs, seed=seed)
+        runner = make_runner(folder, dtype, block, max(peak, max(r64(len(t)) for t in reqs.values())))
+        for st in (steps, traces.portions(reqs), traces.whole(reqs)):
+            worst = check(replay(runner, st), st, ref, TOL[dtype])
+            assert all_free(runner)
+        print(f"seed {seed} {dtype}: worst {worst:.2e}")
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_captured_steps(dtype, tmp_path_factory):
     """The same cuttings with every step as a HIP graph of its shape (padding tokens, requests and
