@@ -76,7 +76,7 @@ def random_config(seed):
     counts and sizes, window, rotated dims, time-mix shape, rank and feed-forward."""
     import random
     rng = random.Random(seed)
-    width = rng.choice([64, 96, 128, 192, 320])
+    width = rng.choice([64, 96, 128, 192, 256])
     vocab = rng.randrange(90, 700)
     layers = []
     for _ in range(rng.randrange(2, 5)):
